@@ -11,6 +11,7 @@ from ..engine.tokenizer import Tokenizer, bert_byte_tokenizer, load_tokenizer, l
 from .bert import BertConfig, BertModel
 from .clip import ClipConfig, ClipModel
 from .decoder_reranker import DecoderRerankerConfig, DecoderRerankerModel
+from .lituvik import LituvikConfig, LituvikModel
 from .llama import LlamaConfig, LlamaModel
 from .mixtral import MixtralConfig, MixtralModel
 from .mllama import MllamaConfig, MllamaModel
@@ -43,6 +44,10 @@ LLM_PRESETS = {
     "pinavik-1b": ("pinavik-1b", lambda: PinavikConfig.sized(2048, 18, 5632, 16, 128)),
     "tiny-ronavik": ("tiny-ronavik", lambda: RonavikConfig.tiny()),
     "ronavik-1b": ("ronavik-1b", lambda: RonavikConfig.sized(2048, 12, 1408, 16, 128, experts=8, top=2)),
+    # hybrid of latent attention, constant-decay linear attention and selective state-space layers (tanh norms,
+    # routed + identity + shared experts, looped block)
+    "tiny-lituvik": ("tiny-lituvik", lambda: LituvikConfig.tiny()),
+    "lituvik-1b": ("lituvik-1b", lambda: LituvikConfig.sized(2048, 18, 5632, 16, 128)),
     "opt-125m": ("facebook/opt-125m", lambda: OPTConfig.opt_125m()),
     "mixtral-8x7b": ("mistralai/mixtral-8x7b-instruct-v0.1", lambda: MixtralConfig.mixtral_8x7b()),
     "tiny-moe": ("tiny-moe", lambda: MixtralConfig.tiny_moe()),
@@ -84,6 +89,8 @@ def build_llm(preset: str = "llama3-8b", weights: Optional[str] = None, device=N
             m = PinavikModel(PinavikConfig.from_json(weights), device=device, dtype=dtype or torch.bfloat16)
         elif arch == "ronavik":
             m = RonavikModel(RonavikConfig.from_json(weights), device=device, dtype=dtype or torch.bfloat16)
+        elif arch == "lituvik":
+            m = LituvikModel(LituvikConfig.from_json(weights), device=device, dtype=dtype or torch.bfloat16)
         elif arch == "opt":
             m = OPTModel(OPTConfig.from_hf(weights), device=device)
         elif arch == "mixtral":
@@ -120,6 +127,9 @@ def build_llm(preset: str = "llama3-8b", weights: Optional[str] = None, device=N
         vocab = cfg.vocab_size
     elif isinstance(cfg, RonavikConfig):
         m = RonavikModel(cfg, device=device, dtype=dtype or torch.bfloat16).random_init(seed)
+        vocab = cfg.vocab_size
+    elif isinstance(cfg, LituvikConfig):
+        m = LituvikModel(cfg, device=device, dtype=dtype or torch.bfloat16).random_init(seed)
         vocab = cfg.vocab_size
     else:
         m = LlamaModel(cfg, device=device).random_init(seed)

@@ -826,17 +826,24 @@ def decode_advance(toks, ids, pos, ctx, slots, block_tables, n_valid):
     native().decode_advance(toks, ids, pos, ctx, slots, block_tables, n_valid, BLOCK)
 
 
-def moe_route(logits: torch.Tensor, k: int, renorm: bool = True, score: str = "softmax"):
+def moe_route(logits: torch.Tensor, k: int, renorm: bool = True, score: str = "softmax", bias=None,
+              eps: float = 0.0):
     """Router scores + top-k -> (expert ids int32 [T,k], weights fp32 [T,k]). score "softmax" (weights optionally
-    renormalised over the chosen experts) or "sigmoid" (each expert scored alone; weights are the chosen scores)."""
+    renormalised over the chosen experts) or "sigmoid" (each expert scored alone; weights are the chosen scores).
+    bias (fp32 [E], softmax scoring): the experts are chosen by score + bias while the weights stay the plain scores;
+    eps is added to the sum that renormalises them."""
     if score not in ("softmax", "sigmoid"):
         raise ValueError(f"moe_route: unknown score function {score!r}")
+    if bias is not None and score != "softmax":
+        raise ValueError("moe_route: a choice bias goes with softmax scoring")
     if not logits.is_cuda:
+        if bias is not None:
+            return ref.moe_route_biased(logits, k, bias, eps)
         return ref.moe_route_sigmoid(logits, k) if score == "sigmoid" else ref.moe_route(logits, k, renorm)
     T = logits.shape[0]
     ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
     w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
-    native().moe_route(logits.float().contiguous(), k, renorm, ids, w, score == "sigmoid")
+    native().moe_route(logits.float().contiguous(), k, renorm, ids, w, score == "sigmoid", bias, float(eps))
     return ids, w
 
 
@@ -958,7 +965,8 @@ _MOE_ACT = {None: 0, "swiglu": 1, "relu2": 2}
 def moe_gemm(A, a_rows, W, offs, rows_total: int, swiglu: bool = False, act: Optional[str] = None):
     """Grouped expert GEMM over expert-sorted rows (A rows gathered through a_rows when given). act: None, "swiglu"
     (W rows interleaved [gate16 | up16]) or "relu2" (squared ReLU). bf16 operands with K % 64 == 0 run on the MFMA
-    tiles; fp32 operands and other shapes on the generic grouped kernel (true fp32 arithmetic)."""
+    tiles; fp32 operands and other shapes on the generic grouped kernel (true fp32 arithmetic). offs may list more
+    groups than W has experts: rows past offs[E] belong to experts without weights and are left untouched."""
     act = "swiglu" if swiglu else act
     if not A.is_cuda:
         return ref.moe_gemm(A, a_rows, W, offs, rows_total, True) if act == "swiglu" else \
@@ -980,12 +988,18 @@ def moe_scale_rows(h, pos, w):
     return out
 
 
-def moe_combine(Y, pos, w, residual=None):
-    """out[t] = sum_j w[t, j] * Y[pos[t, j]] (+ residual); w None: plain sum (the weights were applied upstream)."""
-    if not Y.is_cuda:
+def moe_combine(Y, pos, w, residual=None, ids=None, n_real: int = 0, identity=None):
+    """out[t] = sum_j w[t, j] * Y[pos[t, j]] (+ residual); w None: plain sum (the weights were applied upstream).
+    With ids / n_real / identity: a chosen expert id >= n_real is an identity expert whose output is the token's own
+    row identity[t] (its row of Y is not read)."""
+    if not pos.is_cuda:
+        if ids is not None:
+            return ref.moe_combine_identity(Y, pos, w, residual, ids, n_real, identity)
         return ref.moe_combine(Y, pos, w, residual)
-    out = torch.empty(pos.shape[0], Y.shape[1], dtype=Y.dtype, device=Y.device)
-    native().moe_combine(Y, pos, w, residual, out)
+    D = identity.shape[1] if identity is not None else Y.shape[1]
+    dt = identity.dtype if identity is not None else Y.dtype
+    out = torch.empty(pos.shape[0], D, dtype=dt, device=pos.device)
+    native().moe_combine(Y, pos, w, residual, out, ids, int(n_real), identity)
     return out
 
 
@@ -1290,4 +1304,80 @@ def delta_scan(q, k, v, decay, beta, state, cu, slots, G: int):
     H, DV = state.shape[1], state.shape[3]
     out = torch.empty(v.shape[0], H, DV, dtype=torch.float32, device=v.device)
     native().delta_scan(q, k, v, decay, beta, state, cu, slots, out, G)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# statistics-free tanh norm, latent key / value cache with a partly rotated key, constant-decay linear attention,
+# selective state-space scan
+# ---------------------------------------------------------------------------------------------
+def add_dyt_f32(res: torch.Tensor, delta: Optional[torch.Tensor], extra: Optional[torch.Tensor], alpha: float,
+                w: Optional[torch.Tensor], b: Optional[torch.Tensor], out_dtype=None):
+    """fp32 residual ``res`` (in place) += delta (+ extra, a second fp32 stream such as a re-injected embedding), then
+    (out_dtype given) the dynamic-tanh norm tanh(alpha * res) * w + b in out_dtype: a norm without mean or variance,
+    fused with the residual add of the block before it."""
+    if not res.is_cuda:
+        return ref.add_dyt_f32(res, delta, extra, alpha, w, b, out_dtype)
+    out = torch.empty(res.shape, dtype=out_dtype, device=res.device) if out_dtype is not None else None
+    native().add_dyt_f32(res, delta, extra, float(alpha), w, b, out)
+    return out
+
+
+_ACT_MUL = {"silu": 0, "relu2": 1, "tanh_cap": 2}
+
+
+def act_mul(a: torch.Tensor, b: Optional[torch.Tensor] = None, act: str = "silu", out_dtype=None, cap: float = 0.0):
+    """act(a) (* b) element by element in fp32: "silu", "relu2" (squared ReLU), "tanh_cap" (cap * tanh(a / cap)).
+    a / b may be column slices of wider rows; the result is contiguous in out_dtype (default: a's)."""
+    if act not in _ACT_MUL:
+        raise ValueError(f"act_mul: unknown activation {act!r}")
+    od = out_dtype or a.dtype
+    if not a.is_cuda:
+        return ref.act_mul(a, b, act, od, cap)
+    out = torch.empty(a.shape, dtype=od, device=a.device)
+    native().act_mul(a, b, _ACT_MUL[act], float(cap), out)
+    return out
+
+
+yarn_inv_freq = ref.yarn_inv_freq
+
+
+def latent_kv_write(q, dkv, norm_w, inv_freq, mag: float, positions, slots, q_cat, k_cache, v_cache, H: int, DN: int,
+                    DR: int, R: int, eps: float) -> None:
+    """Cache write of latent attention: the token's latent c = rmsnorm(dkv[:, :R]) * norm_w and its rotated key part
+    kr = rot(dkv[:, R:R + DR]) are the whole cache row - K page row [c | kr] (one kv head of key size R + DR), V^T
+    page c - and the rotated part of every query head (q [T, H * (DN + DR)], the last DR channels of each head) lands
+    in q_cat[:, h, R:] (q_cat [T, H * (R + DR)]; its first R channels per head hold the query folded through the key
+    expansion). The rotation pairs channel i with i + DR / 2 and turns by positions * inv_freq[i]; cos and sin are
+    multiplied by mag (see yarn_inv_freq). Angles, cos / sin and the norm are fp32."""
+    if not q.is_cuda:
+        return ref.latent_kv_write(q, dkv, norm_w, inv_freq, mag, positions, slots, q_cat, k_cache, v_cache, H, DN, DR,
+                                   R, eps)
+    native().latent_kv_write(q, dkv, norm_w, inv_freq, float(mag), positions, slots, q_cat, k_cache, v_cache, H, DN, DR,
+                             R, float(eps))
+
+
+def linear_attention_scan(q, k, v, decay, state, cu, slots):
+    """Linear attention with one constant decay per head: S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t.
+    q / k [T, H * DK], v [T, H * DV]: fp32 column slices of one buffer; decay fp32 [H]; state [slots, H, DK, DV] fp32
+    in place -> fp32 [T, H, DV]. Runs on the state-space scan kernels (step size one, no skip term)."""
+    if not q.is_cuda:
+        return ref.linear_attention_scan(q, k, v, decay, state, cu, slots)
+    H, N, DV = state.shape[1], state.shape[2], state.shape[3]
+    out = torch.empty(q.shape[0], H, DV, dtype=torch.float32, device=q.device)
+    nws = native().ssd_scan_ws_floats(q.shape[0], slots.numel(), H, N, DV)
+    ws = torch.empty(nws, dtype=torch.float32, device=q.device) if nws else None
+    native().linear_attention_scan(q, k, v, decay, state, cu, slots, out, ws)
+    return out
+
+
+def selective_scan(x, dt, dt_bias, A, B, C, D, z, state, cu, slots, out_dtype):
+    """Selective state-space scan with a decay per channel and state element: S[c, n] <- exp(dt_c A[c, n]) S[c, n] +
+    dt_c x_c B_n, y_c = sum_n S[c, n] C_n + D_c x_c, output y * silu(z). dt_c = softplus(dt + dt_bias). x fp32
+    [T, I]; dt fp32 [T, I]; B / C [T, N] and z [T, I] column slices in the activation dtype; A fp32 [I, N] (negative);
+    state [slots, I, N] fp32 in place -> [T, I] in out_dtype. All arithmetic fp32."""
+    if not x.is_cuda:
+        return ref.selective_scan(x, dt, dt_bias, A, B, C, D, z, state, cu, slots, out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    native().selective_scan(x, dt, dt_bias, A, B, C, D, z, state, cu, slots, out)
     return out

@@ -749,3 +749,137 @@ def moe_gemm_act(A, a_rows, W, offs, rows_total, act):
                 y = torch.relu(y) ** 2
             C[o[e]:o[e + 1]] = y.to(A.dtype)
     return C
+
+
+# ---------------------------------------------------------------------------------------------
+# statistics-free tanh norm, latent (low-rank) key / value cache with a partly rotated key, constant-decay linear
+# attention, selective state-space scan, biased top-k routing with identity experts
+# ---------------------------------------------------------------------------------------------
+def add_dyt_f32(res, delta, extra, alpha, w, b, out_dtype):
+    """res (fp32, in place) += delta (+ extra); returns tanh(alpha res) * w + b as out_dtype (None: nothing)."""
+    if delta is not None:
+        res.add_(delta.float())
+    if extra is not None:
+        res.add_(extra.float())
+    if out_dtype is None:
+        return None
+    return (torch.tanh(float(alpha) * res) * w.float() + b.float()).to(out_dtype)
+
+
+def act_mul(a, b, act, out_dtype, cap=0.0):
+    """act(a) (* b): "silu", "relu2" (squared ReLU) or "tanh_cap" (cap tanh(a / cap)), in fp32."""
+    x = a.float()
+    if act == "silu":
+        y = F.silu(x)
+    elif act == "relu2":
+        y = torch.relu(x) ** 2
+    else:
+        y = float(cap) * torch.tanh(x / float(cap))
+    if b is not None:
+        y = y * b.float()
+    return y.to(out_dtype)
+
+
+def yarn_inv_freq(dims, base, scaling=None):
+    """(fp32 [dims / 2] angle steps per position, magnitude of cos / sin) of a rotation over `dims` channels with the
+    pairs (i, i + dims / 2); scaling {factor, original, fast, slow}: wavelengths longer than original / slow are
+    stretched by factor, shorter than original / fast kept, a linear ramp over the pair index between them."""
+    half = dims // 2
+    i = torch.arange(half, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    mag = 1.0
+    if scaling:
+        import math
+
+        fac, orig = float(scaling["factor"]), float(scaling["original"])
+        at = lambda turns: dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))  # noqa: E731
+        lo = max(math.floor(at(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(at(float(scaling["slow"]))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / fac * ramp + f * (1.0 - ramp)
+        mag = 0.1 * math.log(fac) + 1.0
+    return f.to(torch.float32), float(mag)
+
+
+def _rot_half(x, pos, inv_freq, mag):
+    """x [T, ..., dims] fp32, pos [T]; pair (i, i + dims / 2) turned by pos * inv_freq[i], cos / sin times mag."""
+    half = inv_freq.numel()
+    a = pos.float().reshape(-1, *([1] * (x.dim() - 1))) * inv_freq.float()
+    c, s = torch.cos(a) * mag, torch.sin(a) * mag
+    u, v = x[..., :half], x[..., half:2 * half]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., 2 * half:]], -1)
+
+
+def latent_kv_write(q, dkv, norm_w, inv_freq, mag, positions, slots, q_cat, k_cache, v_cache, H, DN, DR, R, eps):
+    """One low-rank latent per token as the only cache row: c = rmsnorm(dkv[:, :R]) * norm_w, kr = rot(dkv[:, R:]).
+    K page row = [c | kr] (one kv head, key size R + DR), V^T page = c. The rotated part of every query head
+    (q [T, H, DN + DR], last DR channels) goes to q_cat[:, h, R:]."""
+    T = q.shape[0]
+    pos = positions[:T]
+    x = dkv.float()
+    c = x[:, :R]
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+    kr = _rot_half(x[:, R:R + DR], pos, inv_freq, mag)
+    s = slots[:T].long()
+    k_cache[s // BLOCK, 0, s % BLOCK] = torch.cat([c, kr], -1).to(k_cache.dtype)
+    v_cache[s // BLOCK, 0, :, s % BLOCK] = c.to(v_cache.dtype)
+    qr = _rot_half(q.float().reshape(T, H, DN + DR)[:, :, DN:], pos, inv_freq, mag)
+    q_cat.view(T, H, R + DR)[:, :, R:] = qr.to(q_cat.dtype)
+
+
+def linear_attention_scan(q, k, v, decay, state, cu, slots):
+    """S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t; q / k [T, H * DK], v [T, H * DV] fp32; state
+    [slots, H, DK, DV] fp32 in place -> fp32 [T, H, DV]."""
+    H, DK, DV = state.shape[1:]
+    T = q.shape[0]
+    q3, k3, v3 = q.float().reshape(T, H, DK), k.float().reshape(T, H, DK), v.float().reshape(T, H, DV)
+    d = decay.float().reshape(H, 1, 1)
+    out = torch.empty(T, H, DV)
+    for lo, hi, s in _seqs(cu, slots):
+        S = state[s]
+        for t in range(lo, hi):
+            S = d * S + k3[t][:, :, None] * v3[t][:, None, :]
+            out[t] = torch.einsum("hkv,hk->hv", S, q3[t])
+        if hi > lo:
+            state[s] = S
+    return out
+
+
+def selective_scan(x, dt, dt_bias, A, B, C, D, z, state, cu, slots, out_dtype):
+    """Selective state-space scan: per channel c and state n, S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n,
+    y_c = sum_n S[c, n] C_n + D_c x_c, times silu(z_c); dt = softplus(dt + dt_bias). x [T, I] fp32, dt [T, I],
+    B / C [T, N], A [I, N] (negative), state [slots, I, N] fp32 in place -> [T, I] in out_dtype."""
+    T, I = x.shape
+    xs = x.float()
+    dts = F.softplus(dt.float() + dt_bias.float().reshape(1, -1))
+    Bf, Cf, Af = B.float(), C.float(), A.float()
+    y = torch.empty(T, I)
+    for lo, hi, s in _seqs(cu, slots):
+        S = state[s]
+        for t in range(lo, hi):
+            S = torch.exp(dts[t][:, None] * Af) * S + (dts[t] * xs[t])[:, None] * Bf[t][None, :]
+            y[t] = S @ Cf[t] + D.float() * xs[t]
+        if hi > lo:
+            state[s] = S
+    return (y * F.silu(z.float())).to(out_dtype)
+
+
+def moe_route_biased(logits, k, bias, eps):
+    """softmax scores s; the k experts with the largest s + bias are chosen; weights s / (sum of the chosen s + eps)."""
+    s = torch.softmax(logits.float(), -1)
+    ids = torch.topk(s + bias.float(), k, dim=-1).indices
+    w = torch.gather(s, 1, ids)
+    return ids.int(), w / (w.sum(-1, keepdim=True) + eps)
+
+
+def moe_combine_identity(Y, pos, w, residual, ids, n_real, h):
+    """moe_combine where an expert id >= n_real is an identity expert: its output is the token's own input row."""
+    T, k = pos.shape
+    rows = Y.float()[pos.reshape(-1).long().clamp(0, max(Y.shape[0] - 1, 0))].reshape(T, k, -1) if Y.shape[0] else \
+        torch.zeros(T, k, h.shape[1])
+    ident = (ids >= n_real)[:, :, None]
+    rows = torch.where(ident, h.float()[:, None, :].expand_as(rows), rows)
+    out = (rows * w.float()[:, :, None]).sum(1)
+    if residual is not None:
+        out = out + residual.float()
+    return out.to(h.dtype)
