@@ -367,9 +367,126 @@ void delta_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor&
                  cur_stream());
 }
 
+void add_dyt_f32(Tensor& res, const optional<Tensor>& delta, const optional<Tensor>& extra, double alpha,
+                 const optional<Tensor>& w, const optional<Tensor>& b, const optional<Tensor>& out) {
+  float* r = f32w(res, "res");
+  TORCH_CHECK(res.dim() == 2, "add_dyt_f32: res [T, D]");
+  const int T = res.size(0), D = res.size(1);
+  int dd = 0, od = 0, ldd = 0;
+  if (delta) {
+    dd = act_dt(*delta, "delta");
+    ldd = row_stride(*delta, "delta");
+    TORCH_CHECK(delta->size(0) == T && delta->size(1) == D, "add_dyt_f32: delta shape");
+  }
+  if (extra) TORCH_CHECK(extra->numel() == (int64_t)T * D, "add_dyt_f32: extra shape");
+  if (out) {
+    od = act_dt(*out, "out");
+    TORCH_CHECK(out->is_contiguous() && out->numel() == (int64_t)T * D && w && b && w->numel() == D && b->numel() == D,
+                "add_dyt_f32: out [T, D] needs weight and bias [D]");
+  }
+  TORCH_CHECK(delta || extra || out, "add_dyt_f32: nothing to do");
+  gai_add_dyt_f32(r, delta ? delta->data_ptr() : nullptr, ldd, extra ? f32(*extra, "extra") : nullptr, (float)alpha,
+                  out ? f32(*w, "w") : nullptr, out ? f32(*b, "b") : nullptr, out ? out->data_ptr() : nullptr, T, D, dd,
+                  od, cur_stream());
+}
+
+void act_mul(const Tensor& a, const optional<Tensor>& b, int64_t act, double cap, Tensor& out) {
+  const int di = act_dt(a, "a"), dout = act_dt(out, "out");
+  const int lda = row_stride(a, "a");
+  const int T = a.size(0), C = a.size(1);
+  int ldb = 0;
+  if (b) {
+    same_dt(*b, di, "b");
+    ldb = row_stride(*b, "b");
+    TORCH_CHECK(b->size(0) == T && b->size(1) == C, "act_mul: b shape");
+  }
+  TORCH_CHECK(out.is_contiguous() && out.numel() == (int64_t)T * C, "act_mul: out shape");
+  gai_act_mul(a.data_ptr(), lda, b ? b->data_ptr() : nullptr, ldb, out.data_ptr(), T, C, (int)act, (float)cap, di, dout,
+              cur_stream());
+}
+
+void latent_kv_write(const Tensor& q, const Tensor& dkv, const Tensor& nw, const Tensor& inv_freq, double mag,
+                     const Tensor& positions, const Tensor& slots, Tensor& q_cat, Tensor& k_cache, Tensor& v_cache,
+                     int64_t H, int64_t DN, int64_t DR, int64_t R, double eps) {
+  const int dt = act_dt(q, "q");
+  same_dt(dkv, dt, "dkv");
+  same_dt(q_cat, dt, "q_cat");
+  same_dt(k_cache, dt, "k_cache");
+  same_dt(v_cache, dt, "v_cache");
+  const int ldq = row_stride(q, "q"), ldk = row_stride(dkv, "dkv");
+  const int T = q.size(0);
+  TORCH_CHECK(q.size(1) == H * (DN + DR) && dkv.size(0) == T && dkv.size(1) == R + DR && nw.numel() == R &&
+                  inv_freq.numel() == DR / 2 && DR % 2 == 0 && positions.numel() >= T && slots.numel() >= T &&
+                  q_cat.is_contiguous() && q_cat.numel() == (int64_t)T * H * (R + DR),
+              "latent_kv_write: shapes");
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() && k_cache.size(1) == 1 && k_cache.size(2) == 16 &&
+                  k_cache.size(3) == R + DR && v_cache.dim() == 4 && v_cache.is_contiguous() && v_cache.size(1) == 1 &&
+                  v_cache.size(2) == R && v_cache.size(3) == 16 && v_cache.size(0) == k_cache.size(0),
+              "latent_kv_write: cache pages K [pages, 1, 16, R + DR], V^T [pages, 1, R, 16]");
+  gai_latent_kv_write(q.data_ptr(), ldq, dkv.data_ptr(), ldk, f32(nw, "norm weight"),
+                      DR ? f32(inv_freq, "inv_freq") : nullptr, (float)mag, i32(positions, "positions"),
+                      i32(slots, "slots"), q_cat.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), T, (int)H, (int)DN,
+                      (int)DR, (int)R, (float)eps, dt, cur_stream());
+}
+
+void linear_attention_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& decay, Tensor& state,
+                           const Tensor& cu, const Tensor& slots, Tensor& out, const optional<Tensor>& ws) {
+  TORCH_CHECK(state.dim() == 4, "linear_attention_scan: state [slots, H, DK, DV]");
+  const int H = state.size(1), N = state.size(2), DV = state.size(3), S = slots.numel();
+  auto f32row = [](const Tensor& t, const char* name) {
+    TORCH_CHECK(t.is_cuda() && t.dim() == 2 && t.scalar_type() == at::kFloat && t.stride(1) == 1, name, " must be fp32 rows");
+    return (int)t.stride(0);
+  };
+  const int ld = f32row(v, "v");
+  TORCH_CHECK(f32row(k, "k") == ld && f32row(q, "q") == ld, "linear_attention_scan: q / k / v must be views of one fp32 buffer");
+  const int T = v.size(0);
+  TORCH_CHECK(v.size(1) == H * DV && k.size(0) == T && k.size(1) == H * N && q.size(0) == T && q.size(1) == H * N &&
+                  decay.numel() == H && cu.numel() == S + 1 && out.numel() == (int64_t)T * H * DV,
+              "linear_attention_scan: shapes");
+  float* wsp = nullptr;
+  if (ws) {
+    TORCH_CHECK(ws->is_cuda() && ws->scalar_type() == at::kFloat && ws->is_contiguous() &&
+                    ws->numel() >= ssd_scan_ws_floats(T, S, H, N, DV), "linear_attention_scan: workspace too small");
+    wsp = ws->data_ptr<float>();
+  }
+  gai_ssd_scan(v.data_ptr<float>(), k.data_ptr<float>(), q.data_ptr<float>(), ld, nullptr, 0, nullptr, nullptr, nullptr,
+               f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, T, f32w(out, "out"), H, H, N, DV, 1, wsp,
+               cur_stream(), f32(decay, "decay"));
+}
+
+void selective_scan(const Tensor& x, const Tensor& dt, const Tensor& dt_bias, const Tensor& A, const Tensor& B,
+                    const Tensor& C, const Tensor& D, const Tensor& z, Tensor& state, const Tensor& cu,
+                    const Tensor& slots, Tensor& out) {
+  TORCH_CHECK(state.dim() == 3, "selective_scan: state [slots, I, N]");
+  const int I = state.size(1), N = state.size(2), S = slots.numel(), T = x.size(0);
+  auto f32row = [](const Tensor& t, const char* name) {
+    TORCH_CHECK(t.is_cuda() && t.dim() == 2 && t.scalar_type() == at::kFloat && t.stride(1) == 1, name, " must be fp32 rows");
+    return (int)t.stride(0);
+  };
+  const int ldx = f32row(x, "x"), lddt = f32row(dt, "dt");
+  const int dtt = act_dt(B, "B");
+  same_dt(C, dtt, "C");
+  same_dt(z, dtt, "z");
+  same_dt(out, dtt, "out");
+  TORCH_CHECK(x.size(1) == I && dt.size(0) == T && dt.size(1) == I && dt_bias.numel() == I && A.numel() == (int64_t)I * N &&
+                  B.size(0) == T && B.size(1) == N && C.size(0) == T && C.size(1) == N && D.numel() == I &&
+                  z.size(0) == T && z.size(1) == I && cu.numel() == S + 1 && out.is_contiguous() &&
+                  out.numel() == (int64_t)T * I,
+              "selective_scan: shapes");
+  gai_selective_scan(x.data_ptr<float>(), ldx, dt.data_ptr<float>(), lddt, f32(dt_bias, "dt_bias"), f32(A, "A"),
+                     B.data_ptr(), row_stride(B, "B"), C.data_ptr(), row_stride(C, "C"), f32(D, "D"), z.data_ptr(),
+                     row_stride(z, "z"), f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, out.data_ptr(), I,
+                     I, N, dtt, cur_stream());
+}
+
 }  // namespace
 
 void gai_bind_seq_ops(pybind11::module_& m) {
+  m.def("add_dyt_f32", &add_dyt_f32);
+  m.def("act_mul", &act_mul);
+  m.def("latent_kv_write", &latent_kv_write);
+  m.def("linear_attention_scan", &linear_attention_scan);
+  m.def("selective_scan", &selective_scan);
   m.def("add_rmsnorm_f32", &add_rmsnorm_f32);
   m.def("poly_norm", &poly_norm);
   m.def("head_norm_gate", &head_norm_gate);

@@ -377,12 +377,17 @@ void sim_topk(const Tensor& Q, const Tensor& X, const Tensor& bias, int64_t n_ro
                cur_stream());
 }
 
-void moe_route(const Tensor& logits, int64_t k, bool renorm, Tensor& ids, Tensor& w, bool sigmoid) {
+void moe_route(const Tensor& logits, int64_t k, bool renorm, Tensor& ids, Tensor& w, bool sigmoid,
+               const optional<Tensor>& bias, double eps) {
   check_f32(logits, "router logits");
   check_i32(ids, "topk ids");
   check_f32(w, "topk weights");
+  if (bias) {
+    check_f32(*bias, "choice bias");
+    TORCH_CHECK(bias->is_contiguous() && bias->numel() == logits.size(1) && !sigmoid, "moe_route: bias [E], softmax scoring");
+  }
   gai_moe_route(logits.data_ptr<float>(), logits.size(0), logits.size(1), k, renorm ? 1 : 0, ids.data_ptr<int>(),
-                w.data_ptr<float>(), cur_stream(), sigmoid ? 1 : 0);
+                w.data_ptr<float>(), cur_stream(), sigmoid ? 1 : 0, bias ? bias->data_ptr<float>() : nullptr, (float)eps);
 }
 
 void moe_scale_rows(const Tensor& h, const Tensor& pos, const Tensor& w, Tensor& out) {
@@ -532,8 +537,15 @@ void moe_dispatch(const Tensor& ids, int64_t E, Tensor& a_rows, Tensor& offs, Te
 }
 
 void moe_combine(const Tensor& Y, const Tensor& pos, const optional<Tensor>& w, const optional<Tensor>& residual,
-                 Tensor& out) {
-  const bool f32 = Y.scalar_type() == at::kFloat;
+                 Tensor& out, const optional<Tensor>& ids, int64_t n_real, const optional<Tensor>& ident) {
+  const bool f32 = out.scalar_type() == at::kFloat;
+  TORCH_CHECK(Y.scalar_type() == out.scalar_type(), "moe_combine: Y / out dtypes differ");
+  if (ids) {
+    check_i32(*ids, "ids");
+    TORCH_CHECK(ident && ident->scalar_type() == out.scalar_type() && ident->is_contiguous() &&
+                    ident->numel() == out.numel() && ids->is_contiguous() && ids->numel() == pos.numel(),
+                "moe_combine: identity experts need ids [T, k] and the input rows [T, D]");
+  }
   if (f32) {
     check_f32(Y, "Y");
     check_f32(out, "out");
@@ -547,8 +559,10 @@ void moe_combine(const Tensor& Y, const Tensor& pos, const optional<Tensor>& w, 
   const int T = pos.size(0), k = pos.size(1), D = out.size(-1);
   TORCH_CHECK(Y.is_contiguous() && out.is_contiguous() && pos.is_contiguous() && Y.size(-1) == D &&
                   (!w || (w->is_contiguous() && w->numel() == pos.numel())), "moe_combine: shapes");
+  if (residual) TORCH_CHECK(residual->is_contiguous() && residual->numel() == out.numel(), "moe_combine: residual shape");
   gai_moe_combine(Y.data_ptr(), pos.data_ptr<int>(), w ? w->data_ptr<float>() : nullptr, opt_ptr(residual),
-                  out.data_ptr(), T, k, D, cur_stream(), f32 ? 1 : 0);
+                  out.data_ptr(), T, k, D, cur_stream(), f32 ? 1 : 0, ids ? ids->data_ptr<int>() : nullptr, (int)n_real,
+                  ident ? ident->data_ptr() : nullptr);
 }
 
 void embedding(const Tensor& ids, const Tensor& table, Tensor& out, int64_t vstart, int64_t vend) {

@@ -142,13 +142,14 @@ int gai_moe_gemm_dec2(const void* A, const int* a_rows, const void* W, void* C, 
                       int rows_total, int N, int K, int act, hipStream_t st);
 // sigmoid: scores sigmoid(logit) per expert instead of a softmax over the experts (weights = the chosen scores)
 void gai_moe_route(const float* logits, int T, int E, int k, int renorm, int* ids, float* w, hipStream_t st,
-                   int sigmoid = 0);
+                   int sigmoid = 0, const float* bias = nullptr, float eps = 0.f);
 // dt: 0 bf16 (MFMA tiles when K % 64 == 0), 1 fp32 (generic grouped kernel, true fp32)
 void gai_moe_gemm(const void* A, const int* a_rows, const void* W, void* C, const int* offs, int E, int rows_total,
                   int N, int K, int act, hipStream_t st, int dt = 0);
 // w = nullptr: plain sum of the k rows
 void gai_moe_combine(const void* Y, const int* pos, const float* w, const void* residual, void* out, int T, int k,
-                     int D, hipStream_t st, int dt = 0);
+                     int D, hipStream_t st, int dt = 0, const int* ids = nullptr, int n_real = 0,
+                     const void* ident = nullptr);
 void gai_moe_scale_rows(const void* h, const int* pos, const float* w, void* out, int T, int k, int D, int dt,
                         hipStream_t st);
 
@@ -220,6 +221,15 @@ void gai_gated_norm_add_f32(float* res, const void* y, int ldy, int dt_y, const 
                             hipStream_t st);
 void gai_gate_group_norm(const float* y, const void* z, int ldz, const float* w, void* out, int T, int NG, int GS,
                          float eps, int dt, hipStream_t st);
+// res += delta (+ extra); out = tanh(alpha res) * w + b (out may be null)
+void gai_add_dyt_f32(float* res, const void* delta, int ldd, const float* extra, float alpha, const float* w,
+                     const float* b, void* out, int T, int D, int dt_delta, int dt_out, hipStream_t st);
+// out = act(a) (* b): act 0 silu, 1 squared ReLU, 2 cap * tanh(a / cap)
+void gai_act_mul(const void* a, int lda, const void* b, int ldb, void* out, int T, int C, int act, float cap, int dt_in,
+                 int dt_out, hipStream_t st);
+void gai_latent_kv_write(const void* q, int ldq, const void* dkv, int ldk, const float* nw, const float* inv_freq,
+                         float mag, const int* positions, const int* slots, void* q_cat, void* k_cache, void* v_cache,
+                         int T, int H, int DN, int DR, int R, float eps, int dt, hipStream_t st);
 // attention_window.hip
 void gai_qknorm_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* wq,
                          const float* wk, const int* slots, void* q_out, void* k_cache, void* v_cache, int T, int H,
@@ -253,7 +263,12 @@ void gai_rglru_scan(const float* a, const float* b, const void* y, int ldy, floa
 void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const void* dt, int lddt,
                   const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu,
                   const int* slots, int S, int T, float* out, int H, int G, int N, int DV, int dtt, float* ws,
-                  hipStream_t st);
+                  hipStream_t st, const float* fixed = nullptr);
+// decay per channel and state element; x / dt fp32, B / C / z / out bf16 (dtt 0) or fp32 (dtt 1)
+void gai_selective_scan(const float* x, int ldx, const float* dt, int lddt, const float* dt_bias, const float* A,
+                        const void* B, int ldb, const void* C, int ldc, const float* D, const void* z, int ldz,
+                        float* state, const int* cu, const int* slots, int S, void* out, int ldo, int I, int N, int dtt,
+                        hipStream_t st);
 // scratch (fp32 elements) for the chunk-parallel form of a step with long portions of few sequences; 0: not chunked
 size_t gai_ssd_scan_ws_floats(int T, int S, int H, int N, int DV);
 void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,

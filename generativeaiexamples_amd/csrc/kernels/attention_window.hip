@@ -20,6 +20,13 @@
 // qknorm_kv_write: RMS norm over the WHOLE q projection (all heads at once) and over the whole k projection, each
 // with its own weight vector, then q -> q_out and k, v -> their cache slots: one pass over the token's rows.
 //
+// latent_kv_write: the cache write of latent attention. A token's cache row is ONE low-rank latent c = rmsnorm(first R
+// channels of the down projection) * w plus DR rotated key channels shared by all heads: K page row [c | kr] (one kv
+// head, key size R + DR), V^T page c. The rotated DR channels of every query head go to the tail of that head's row of
+// q_cat (whose first R channels hold the query folded through the key expansion), so window_attention scores against
+// the cached row directly. Rotation: channel i pairs with i + DR / 2, angle = position * inv_freq[i] (fp32, libm
+// sincosf), cos and sin times one magnitude.
+//
 // window_attention, row kernel: one wave64 per (token, head) (a sequence is (cu_q[s], ctx[s]); the query at row t has
 // position ctx - q_len + (t - cu_q)). Keys are walked in page-aligned blocks of 64: lane j scores key j (q broadcast
 // from LDS, the K row read with 16-byte loads), an online softmax keeps (m, l) per wave, then lane c accumulates output
@@ -166,6 +173,57 @@ __global__ __launch_bounds__(256) void headnorm_kv_write_kernel(const TA* __rest
   for (int i = threadIdx.x; i < NV; i += 256) {
     const int g = i / DV, c = i - g * DV;
     v_cache[((page * G + g) * DV + c) * 16 + off] = vr[i];
+  }
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void latent_kv_write_kernel(const TA* __restrict__ q, int ldq, const TA* __restrict__ dkv,
+                                                              int ldk, const float* __restrict__ nw,
+                                                              const float* __restrict__ inv_freq, float mag,
+                                                              const int* __restrict__ positions,
+                                                              const int* __restrict__ slots, TA* __restrict__ q_cat,
+                                                              TA* __restrict__ k_cache, TA* __restrict__ v_cache, int H,
+                                                              int DN, int DR, int R, float eps) {
+  extern __shared__ float cs[];  // cos[DR / 2] | sin[DR / 2]
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, tid = threadIdx.x, half = DR >> 1;
+  const TA* lr = dkv + (size_t)t * ldk;
+  const float pos = (float)positions[t];
+  for (int i = tid; i < half; i += 256) {
+    float sn, c;
+    sincosf(pos * inv_freq[i], &sn, &c);
+    cs[i] = c * mag;
+    cs[half + i] = sn * mag;
+  }
+  float ss = 0.f;
+  for (int i = tid; i < R; i += 256) {
+    const float x = (float)lr[i];
+    ss += x * x;
+  }
+  ss = block_sum(ss, scratch);  // also orders the cos / sin table before its readers
+  __syncthreads();
+  const float inv = 1.0f / sqrtf(ss / R + eps);
+  const int slot = slots[t];
+  const size_t page = slot >> 4;
+  const int off = slot & 15, DK = R + DR;
+  TA* kr = k_cache + (page * 16 + off) * DK;
+  for (int i = tid; i < R; i += 256) {
+    const TA c = (TA)((float)lr[i] * inv * nw[i]);
+    kr[i] = c;
+    v_cache[(page * R + i) * 16 + off] = c;
+  }
+  for (int i = tid; i < half; i += 256) {
+    const float u = (float)lr[R + i], v = (float)lr[R + half + i], c = cs[i], sn = cs[half + i];
+    kr[R + i] = (TA)(u * c - v * sn);
+    kr[R + half + i] = (TA)(v * c + u * sn);
+  }
+  for (int x = tid; x < H * half; x += 256) {
+    const int h = x / half, i = x - h * half;
+    const TA* qr = q + (size_t)t * ldq + (size_t)h * (DN + DR) + DN;
+    TA* qo = q_cat + ((size_t)t * H + h) * DK + R;
+    const float u = (float)qr[i], v = (float)qr[half + i], c = cs[i], sn = cs[half + i];
+    qo[i] = (TA)(u * c - v * sn);
+    qo[half + i] = (TA)(v * c + u * sn);
   }
 }
 
@@ -484,6 +542,23 @@ void gai_headnorm_kv_write(const void* q, int ldq, const void* k, int ldk, const
     headnorm_kv_write_kernel<bf16><<<T, 256, 0, st>>>((const bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv, wq,
                                                       wk, slots, positions, (bf16*)q_out, (bf16*)k_cache,
                                                       (bf16*)v_cache, H, G, DK, DV, eps, temp_coef, temp_every);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_latent_kv_write(const void* q, int ldq, const void* dkv, int ldk, const float* nw, const float* inv_freq,
+                         float mag, const int* positions, const int* slots, void* q_cat, void* k_cache, void* v_cache,
+                         int T, int H, int DN, int DR, int R, float eps, int dt, hipStream_t st) {
+  if (T == 0) return;
+  if (DR % 2 || R < 1) gai_launch_error(__FILE__, __LINE__, "latent_kv_write: even rotated size, latent size >= 1");
+  const size_t lds = (size_t)(DR > 0 ? DR : 1) * sizeof(float);
+  if (dt)
+    latent_kv_write_kernel<float><<<T, 256, lds, st>>>((const float*)q, ldq, (const float*)dkv, ldk, nw, inv_freq, mag,
+                                                       positions, slots, (float*)q_cat, (float*)k_cache,
+                                                       (float*)v_cache, H, DN, DR, R, eps);
+  else
+    latent_kv_write_kernel<bf16><<<T, 256, lds, st>>>((const bf16*)q, ldq, (const bf16*)dkv, ldk, nw, inv_freq, mag,
+                                                      positions, slots, (bf16*)q_cat, (bf16*)k_cache, (bf16*)v_cache, H,
+                                                      DN, DR, R, eps);
   GAI_LAUNCH_CHECK();
 }
 

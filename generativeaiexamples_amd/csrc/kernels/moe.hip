@@ -14,6 +14,9 @@
 // moe_combine: out[t] = sum_j w[t, j] * Y[pos[t, j]] (+ residual), bf16x8 vectorised (generic kernel: fp32 rows, any
 //              width, w optional).
 // moe_route (sigmoid): every expert scored alone by sigmoid(logit); the weights are the chosen scores.
+// moe_route (choice bias): the experts are chosen by softmax score + bias_e while the weights stay the plain scores,
+//              renormalised over the chosen ones (+ eps in the sum); libm expf, all fp32.
+// moe_combine (identity experts): a chosen id >= n_real has no weights - its output is the token's own input row.
 // moe_scale_rows: expert-sorted copies of the token rows, each times its routing weight (experts whose routing weight
 //              multiplies the INPUT of a non-linear expert).
 #include "gai_common.h"
@@ -27,15 +30,20 @@ constexpr int MBM = 128, MBN = 128, MBK = 64;
 constexpr int kMTile = MBM * MBK * 2;
 
 __global__ void moe_route_kernel(const float* __restrict__ logits, int T, int E, int k, int renorm,
-                                 int* __restrict__ ids, float* __restrict__ w, int sigmoid) {
+                                 int* __restrict__ ids, float* __restrict__ w, int sigmoid,
+                                 const float* __restrict__ bias, float eps) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const float* x = logits + (size_t)t * E;
   float mx = -INFINITY;
   for (int e = 0; e < E; ++e) mx = fmaxf(mx, x[e]);
   float s = 0.f;
-  if (!sigmoid)
-    for (int e = 0; e < E; ++e) s += __expf(x[e] - mx);
+  if (!sigmoid) {
+    if (bias)
+      for (int e = 0; e < E; ++e) s += expf(x[e] - mx);
+    else
+      for (int e = 0; e < E; ++e) s += __expf(x[e] - mx);
+  }
   float bv[8];
   int bi[8];
   for (int j = 0; j < k; ++j) {
@@ -43,7 +51,8 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int T, int E,
     bi[j] = 0;
   }
   for (int e = 0; e < E; ++e) {
-    const float p = sigmoid ? 1.0f / (1.0f + expf(-x[e])) : __expf(x[e] - mx) / s;
+    float p = sigmoid ? 1.0f / (1.0f + expf(-x[e])) : (bias ? expf(x[e] - mx) : __expf(x[e] - mx)) / s;
+    if (bias) p += bias[e];  // the choice is made on the corrected score
     if (p > bv[k - 1]) {
       int j = k - 1;
       while (j > 0 && bv[j - 1] < p) {
@@ -55,7 +64,9 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int T, int E,
       bi[j] = e;
     }
   }
-  float tot = 0.f;
+  if (bias)
+    for (int j = 0; j < k; ++j) bv[j] = expf(x[bi[j]] - mx) / s;  // the weights are the plain scores
+  float tot = eps;
   for (int j = 0; j < k; ++j) tot += bv[j];
   for (int j = 0; j < k; ++j) {
     ids[(size_t)t * k + j] = bi[j];
@@ -244,6 +255,13 @@ __global__ __launch_bounds__(256) void moe_gemm_generic_kernel(const TA* __restr
     for (int c = 0; c < 4; ++c) {
       const int n = n0 + tx + 16 * c;
       float v = acc[r][c];
+      if (ACT == 1) {  // rows interleaved [gate16 | up16]: columns c = 0, 2 are gates, c + 1 their up partners
+        if ((c & 1) == 0 && n + 16 < N) {
+          const float g = v;
+          C[(size_t)m * (N / 2) + n0 / 2 + tx + 16 * (c >> 1)] = (TA)(g / (1.0f + expf(-g)) * acc[r][c + 1]);
+        }
+        continue;
+      }
       if (ACT == 2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
       if (n < N) C[(size_t)m * N + n] = (TA)v;
     }
@@ -253,13 +271,16 @@ __global__ __launch_bounds__(256) void moe_gemm_generic_kernel(const TA* __restr
 template <typename TA>
 __global__ __launch_bounds__(256) void moe_combine_generic_kernel(const TA* __restrict__ Y, const int* __restrict__ pos,
                                                                   const float* __restrict__ w, const TA* residual,
-                                                                  TA* __restrict__ out, int T, int k, int D) {
+                                                                  TA* __restrict__ out, int T, int k, int D,
+                                                                  const int* __restrict__ ids, int n_real,
+                                                                  const TA* __restrict__ ident) {
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= (long)T * D) return;
   const int t = (int)(e / D), d = (int)(e % D);
   float acc = 0.f;
   for (int j = 0; j < k; ++j) {
-    const float y = (float)Y[(size_t)pos[(size_t)t * k + j] * D + d];
+    const bool idn = ids && ids[(size_t)t * k + j] >= n_real;
+    const float y = idn ? (float)ident[(size_t)t * D + d] : (float)Y[(size_t)pos[(size_t)t * k + j] * D + d];
     acc += w ? w[(size_t)t * k + j] * y : y;
   }
   if (residual) acc += (float)residual[(size_t)t * D + d];
@@ -279,7 +300,9 @@ __global__ __launch_bounds__(256) void moe_scale_rows_kernel(const TA* __restric
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(const bf16* __restrict__ Y, const int* __restrict__ pos,
                                                           const float* __restrict__ w, const bf16* residual,
-                                                          bf16* __restrict__ out, int T, int k, int D) {
+                                                          bf16* __restrict__ out, int T, int k, int D,
+                                                          const int* __restrict__ ids, int n_real,
+                                                          const bf16* __restrict__ ident) {
   const int units = D / 8;
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= (long)T * units) return;
@@ -287,7 +310,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const bf16* __restrict
   float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   for (int j = 0; j < k; ++j) {
     const float wj = w[(size_t)t * k + j];
-    const bf16x8 y = load8(Y + (size_t)pos[(size_t)t * k + j] * D + u * 8);
+    const bool idn = ids && ids[(size_t)t * k + j] >= n_real;
+    const bf16x8 y = load8(idn ? ident + (size_t)t * D + u * 8 : Y + (size_t)pos[(size_t)t * k + j] * D + u * 8);
 #pragma unroll
     for (int q = 0; q < 8; ++q) acc[q] += wj * (float)y[q];
   }
@@ -453,10 +477,10 @@ void gai_moe_dispatch(const int* ids, int n, int k, int E, int* a_rows, int* off
 }
 
 void gai_moe_route(const float* logits, int T, int E, int k, int renorm, int* ids, float* w, hipStream_t st,
-                   int sigmoid) {
+                   int sigmoid, const float* bias, float eps) {
   if (T == 0) return;
   if (k < 1 || k > 8 || k > E) gai_launch_error(__FILE__, __LINE__, "moe_route: 1 <= top-k <= min(8, experts)");
-  moe_route_kernel<<<(T + 255) / 256, 256, 0, st>>>(logits, T, E, k, renorm, ids, w, sigmoid);
+  moe_route_kernel<<<(T + 255) / 256, 256, 0, st>>>(logits, T, E, k, renorm, ids, w, sigmoid, bias, eps);
   GAI_LAUNCH_CHECK();
 }
 
@@ -475,14 +499,14 @@ void gai_moe_gemm(const void* A, const int* a_rows, const void* W, void* C, cons
   if (rows_total == 0) return;
   if (act < 0 || act > 2) gai_launch_error(__FILE__, __LINE__, "moe_gemm: act 0 (none), 1 (SwiGLU) or 2 (squared ReLU)");
   if (dt || K % MBK) {  // fp32 operands, or K off the MFMA tile grid: the generic grouped kernel
-    if (act == 1) gai_launch_error(__FILE__, __LINE__, "moe_gemm: SwiGLU needs bf16 operands with K % 64 == 0");
+    if (act == 1 && N % 32) gai_launch_error(__FILE__, __LINE__, "moe_gemm: SwiGLU rows come in [gate16 | up16] blocks");
     const dim3 grid((rows_total + 31) / 32 + E, (N + 63) / 64);
 #define GAI_MG(TA, ACT_)                                                                                        \
   moe_gemm_generic_kernel<TA, ACT_><<<grid, 256, 0, st>>>((const TA*)A, a_rows, (const TA*)W, (TA*)C, offs, E, N, K)
     if (dt) {
-      if (act == 2) GAI_MG(float, 2); else GAI_MG(float, 0);
+      if (act == 2) GAI_MG(float, 2); else if (act == 1) GAI_MG(float, 1); else GAI_MG(float, 0);
     } else {
-      if (act == 2) GAI_MG(bf16, 2); else GAI_MG(bf16, 0);
+      if (act == 2) GAI_MG(bf16, 2); else if (act == 1) GAI_MG(bf16, 1); else GAI_MG(bf16, 0);
     }
 #undef GAI_MG
     GAI_LAUNCH_CHECK();
@@ -510,21 +534,21 @@ void gai_moe_gemm(const void* A, const int* a_rows, const void* W, void* C, cons
 }
 
 void gai_moe_combine(const void* Y, const int* pos, const float* w, const void* residual, void* out, int T, int k,
-                     int D, hipStream_t st, int dt) {
+                     int D, hipStream_t st, int dt, const int* ids, int n_real, const void* ident) {
   if (T == 0) return;
   if (dt || D % 8 || !w) {
     const long n = (long)T * D;
     if (dt)
       moe_combine_generic_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(
-          (const float*)Y, pos, w, (const float*)residual, (float*)out, T, k, D);
+          (const float*)Y, pos, w, (const float*)residual, (float*)out, T, k, D, ids, n_real, (const float*)ident);
     else
       moe_combine_generic_kernel<bf16><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(
-          (const bf16*)Y, pos, w, (const bf16*)residual, (bf16*)out, T, k, D);
+          (const bf16*)Y, pos, w, (const bf16*)residual, (bf16*)out, T, k, D, ids, n_real, (const bf16*)ident);
     GAI_LAUNCH_CHECK();
     return;
   }
   const long n = (long)T * (D / 8);
   moe_combine_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const bf16*)Y, pos, w, (const bf16*)residual,
-                                                                   (bf16*)out, T, k, D);
+                                                                   (bf16*)out, T, k, D, ids, n_real, (const bf16*)ident);
   GAI_LAUNCH_CHECK();
 }

@@ -9,6 +9,10 @@
 //                     (post-norm gated residual: the closing norm of a sublayer, the residual add and the opening norm
 //                     of the next sublayer in one pass)
 //   gate_group_norm   g = y * silu(z);  out = g * rsqrt(mean_group(g^2) + eps) * w, the row cut into equal groups
+//   add_dyt_f32       res += delta (+ extra);  out = tanh(alpha * res) * w + b   (dynamic tanh: a norm without statistics,
+//                     so the pass is purely element-wise: four elements per thread, no reduction)
+//   act_mul           out = act(a) (* b), act: silu | squared ReLU | cap * tanh(a / cap); fp32 arithmetic, a / b column
+//                     slices of wider rows, out bf16 or fp32
 //
 // Activations (delta, z, gate, out, y) are bf16 or fp32 (template TA); every statistic and product is fp32.
 // One wave64 per row for the row norms (D of a few thousand: the row is re-read from L2 in the second pass).
@@ -287,6 +291,55 @@ __global__ __launch_bounds__(256) void gate_group_norm_kernel(const float* __res
   }
 }
 
+// ---- dynamic tanh norm fused with the residual add --------------------------------------------------------------------
+template <typename TD, typename TA, int VEC>
+__global__ __launch_bounds__(256) void add_dyt_f32_kernel(float* __restrict__ res, const TD* __restrict__ delta, int ldd,
+                                                          const float* __restrict__ extra, float alpha,
+                                                          const float* __restrict__ w, const float* __restrict__ b,
+                                                          TA* __restrict__ out, int T, int D) {
+  const int per = D / VEC;
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long)T * per) return;
+  const int row = (int)(e / per), c0 = (int)(e % per) * VEC;
+  float* r = res + (size_t)row * D + c0;
+  float v[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) v[i] = r[i];
+  if (delta) {
+    const TD* d = delta + (size_t)row * ldd + c0;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] += (float)d[i];
+  }
+  if (extra) {
+    const float* x = extra + (size_t)row * D + c0;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] += x[i];
+  }
+  if (delta || extra) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) r[i] = v[i];
+  }
+  if (!out) return;
+  TA* o = out + (size_t)row * D + c0;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) o[i] = (TA)fmaf(tanhf(alpha * v[i]), w[c0 + i], b[c0 + i]);
+}
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void act_mul_kernel(const TI* __restrict__ a, int lda, const TI* __restrict__ b, int ldb,
+                                                      TO* __restrict__ out, int T, int C, int act, float cap) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long)T * C) return;
+  const int row = (int)(e / C), c = (int)(e % C);
+  const float x = (float)a[(size_t)row * lda + c];
+  float y;
+  if (act == 0) y = x / (1.0f + expf(-x));
+  else if (act == 1) y = fmaxf(x, 0.f) * fmaxf(x, 0.f);
+  else y = cap * tanhf(x / cap);
+  if (b) y *= (float)b[(size_t)row * ldb + c];
+  out[e] = (TO)y;
+}
+
 }  // namespace
 
 void gai_add_rmsnorm_f32(float* res, const void* delta, int ldd, float mult, const float* w, void* out, int T, int D,
@@ -375,5 +428,43 @@ void gai_gate_group_norm(const float* y, const void* z, int ldz, const float* w,
     gate_group_norm_kernel<float><<<grid, 256, 0, st>>>(y, (const float*)z, ldz, w, (float*)out, TG, NG, GS, eps);
   else
     gate_group_norm_kernel<bf16><<<grid, 256, 0, st>>>(y, (const bf16*)z, ldz, w, (bf16*)out, TG, NG, GS, eps);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_add_dyt_f32(float* res, const void* delta, int ldd, const float* extra, float alpha, const float* w,
+                     const float* b, void* out, int T, int D, int dt_delta, int dt_out, hipStream_t st) {
+  if (T == 0) return;
+  const bool v4 = D % 4 == 0 && (!delta || ldd % 4 == 0);
+  const long n = (long)T * (v4 ? D / 4 : D);
+  const unsigned grid = (unsigned)((n + 255) / 256);
+#define GAI_DYT(TD, TA)                                                                                               \
+  do {                                                                                                                \
+    if (v4) add_dyt_f32_kernel<TD, TA, 4><<<grid, 256, 0, st>>>(res, (const TD*)delta, ldd, extra, alpha, w, b,       \
+                                                                (TA*)out, T, D);                                      \
+    else add_dyt_f32_kernel<TD, TA, 1><<<grid, 256, 0, st>>>(res, (const TD*)delta, ldd, extra, alpha, w, b,          \
+                                                             (TA*)out, T, D);                                         \
+  } while (0)
+  if (dt_delta && dt_out) GAI_DYT(float, float);
+  else if (dt_delta) GAI_DYT(float, bf16);
+  else if (dt_out) GAI_DYT(bf16, float);
+  else GAI_DYT(bf16, bf16);
+#undef GAI_DYT
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_act_mul(const void* a, int lda, const void* b, int ldb, void* out, int T, int C, int act, float cap, int dt_in,
+                 int dt_out, hipStream_t st) {
+  if (T == 0 || C == 0) return;
+  if (act < 0 || act > 2) gai_launch_error(__FILE__, __LINE__, "act_mul: act 0 (silu), 1 (squared ReLU) or 2 (tanh cap)");
+  if (act == 2 && !(cap > 0.f)) gai_launch_error(__FILE__, __LINE__, "act_mul: the tanh cap must be positive");
+  const long n = (long)T * C;
+  const unsigned grid = (unsigned)((n + 255) / 256);
+#define GAI_AM(TI, TO) \
+  act_mul_kernel<TI, TO><<<grid, 256, 0, st>>>((const TI*)a, lda, (const TI*)b, ldb, (TO*)out, T, C, act, cap)
+  if (dt_in && dt_out) GAI_AM(float, float);
+  else if (dt_in) GAI_AM(float, bf16);
+  else if (dt_out) GAI_AM(bf16, float);
+  else GAI_AM(bf16, bf16);
+#undef GAI_AM
   GAI_LAUNCH_CHECK();
 }

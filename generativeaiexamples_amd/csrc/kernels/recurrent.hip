@@ -15,7 +15,11 @@
 //   rglru_scan        S <- a_t S + b_t per channel; o_t = scale * S_t * act(y_t)
 //   ssd_scan          state-space scan with one decay per head: S [N, DV], dt_t = softplus(dt + dt_bias),
 //                     S <- exp(-exp(A_log) dt_t) S + dt_t B_t x_t^T;  o_t = S^T C_t + D x_t  (the output reads the
-//                     UPDATED state)
+//                     UPDATED state); with a fixed decay per head, step size one and no skip term it is linear
+//                     attention with a constant decay: S <- decay_h S + k_t v_t^T, o_t = S^T q_t
+//   selective_scan    state-space scan with a decay per channel AND state element, everything input-dependent:
+//                     dt_c = softplus(dt + dt_bias); S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n;
+//                     y_c = sum_n S[c, n] C_n + D_c x_c; out = y * silu(z)
 //
 // A batch is S sequences of rows [cu[s], cu[s+1]) with pool slot slots[s] (device vectors: graph-capturable); a decoded
 // token is a sequence of one row, a prompt portion a longer one. The scans keep the state in VGPRs for the whole
@@ -786,7 +790,7 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(const float* __restrict_
                                                         const float* __restrict__ A_log, const float* __restrict__ Dskip,
                                                         float* __restrict__ state, const int* __restrict__ cu,
                                                         const int* __restrict__ slots, float* __restrict__ out, int H,
-                                                        int G, int N, int DV) {
+                                                        int G, int N, int DV, const float* __restrict__ fixed) {
   extern __shared__ float lds[];  // buf[2][2][N] (B, C) | red[2][RG][DV]
   const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
   const int RG = (N + kRows - 1) / kRows;
@@ -801,7 +805,9 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(const float* __restrict_
   float col[kRows];
 #pragma unroll
   for (int i = 0; i < kRows; ++i) col[i] = i < nrow ? Sg[(size_t)i * DV] : 0.f;
-  const float negA = -expf(A_log[h]), dskip = Dskip[h], dtb = dt_bias[h];
+  // fixed: one constant decay per head, step size one, no skip term (constant-decay linear attention)
+  const float negA = fixed ? 0.f : -expf(A_log[h]), dskip = Dskip ? Dskip[h] : 0.f, dtb = fixed ? 0.f : dt_bias[h];
+  const float fdec = fixed ? fixed[h] : 0.f;
   for (int t = t0; t < t1; ++t) {
     const int b = (t - t0) & 1;
     float* bb = buf + b * 2 * N;
@@ -810,8 +816,8 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(const float* __restrict_
       bb[N + i] = Cm[(size_t)t * ld + (size_t)g * N + i];
     }
     const float xj = x[(size_t)t * ld + (size_t)h * DV + j];
-    const float dtv = softplus_f((float)dt[(size_t)t * lddt + h] + dtb);
-    const float dec = expf(negA * dtv), dx = dtv * xj;
+    const float dtv = fixed ? 1.0f : softplus_f((float)dt[(size_t)t * lddt + h] + dtb);
+    const float dec = fixed ? fdec : expf(negA * dtv), dx = dtv * xj;
     __syncthreads();
     float acc = 0.f;
 #pragma unroll
@@ -855,7 +861,8 @@ __global__ __launch_bounds__(64) void ssd_scan_cols_kernel(const float* __restri
                                                            const float* __restrict__ Dskip, float* __restrict__ state,
                                                            const int* __restrict__ cu, const int* __restrict__ slots,
                                                            float* __restrict__ out, int H, int G, int N, int DV, int S,
-                                                           float* __restrict__ Pbuf, float* __restrict__ Qbuf) {
+                                                           float* __restrict__ Pbuf, float* __restrict__ Qbuf,
+                                                           const float* __restrict__ fixed) {
   constexpr int COLS = 64 / RGS, NP = kTB * RGS * R / 64, LD = RGS * R + RGS;
   extern __shared__ float lds[];
   const int h = blockIdx.x, cb = blockIdx.z, lane = threadIdx.x;
@@ -883,7 +890,8 @@ __global__ __launch_bounds__(64) void ssd_scan_cols_kernel(const float* __restri
   float pprod = 1.f;
 #pragma unroll
   for (int i = 0; i < R; ++i) col[i] = (MODE != 1 && on && i < nrow) ? Sg[(size_t)i * DV] : 0.f;
-  const float negA = -expf(A_log[h]), dskip = Dskip[h], dtb = dt_bias[h];
+  const float negA = fixed ? 0.f : -expf(A_log[h]), dskip = Dskip ? Dskip[h] : 0.f, dtb = fixed ? 0.f : dt_bias[h];
+  const float fdec = fixed ? fixed[h] : 0.f;
   constexpr int NPART = 64 / kTB;
   static_assert(NP * NPART >= RGS * R, "staging covers a full row");
   const int stt = lane / NPART, spart = lane % NPART;
@@ -905,8 +913,8 @@ __global__ __launch_bounds__(64) void ssd_scan_cols_kernel(const float* __restri
       pv[q] = (tt < n && c < DV) ? x[(size_t)(tb + tt) * ld + (size_t)h * DV + c] : 0.f;
     }
     if (lane < n) {
-      pdt = softplus_f((float)dt[(size_t)(tb + lane) * lddt + h] + dtb);
-      pdec = expf(negA * pdt);
+      pdt = fixed ? 1.0f : softplus_f((float)dt[(size_t)(tb + lane) * lddt + h] + dtb);
+      pdec = fixed ? fdec : expf(negA * pdt);
     }
   };
   fetch(t0);
@@ -978,6 +986,75 @@ __global__ __launch_bounds__(256) void ssd_chunk_carry_kernel(const float* __res
     Sv = fmaf(Pbuf[(size_t)(first + n) * H + h], Sv, q);
   }
   *sp = Sv;
+}
+
+// ---- selective state-space scan: a decay per channel and state element ----------------------------------------------
+// Every (channel, state element) pair is its own scalar recurrence, so there is nothing to contract but the N states of
+// a channel at the output: J = 2^k lanes share a channel, each keeping up to PER states in registers (J * PER >= N), and
+// the output sum is a J-lane butterfly. B_t and C_t (shared by all channels) are staged through LDS kST tokens at a
+// time; exp(dt A) runs on the exponent unit with A pre-multiplied by log2(e). The same kernel serves prompt portions and
+// single decoded tokens (a sequence of one row).
+constexpr int kST = 16;
+
+template <typename TA, int PER>
+__global__ __launch_bounds__(256) void selective_scan_kernel(
+    const float* __restrict__ x, int ldx, const float* __restrict__ dt, int lddt, const float* __restrict__ dt_bias,
+    const float* __restrict__ A, const TA* __restrict__ Bm, int ldb, const TA* __restrict__ Cm, int ldc,
+    const float* __restrict__ Dskip, const TA* __restrict__ z, int ldz, float* __restrict__ state,
+    const int* __restrict__ cu, const int* __restrict__ slots, TA* __restrict__ out, int ldo, int I, int N, int J) {
+  extern __shared__ float lds[];  // B[kST][N] | C[kST][N]
+  const int s = blockIdx.y, tid = threadIdx.x;
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;  // uniform over the workgroup
+  float* Bs = lds;
+  float* Cs = lds + kST * N;
+  const int c = blockIdx.x * (256 / J) + tid / J, j = tid % J;
+  const bool on = c < I;
+  const int per = (N + J - 1) / J, n0 = j * per;
+  const int nv = on ? max(0, min(per, N - n0)) : 0;
+  float a2[PER], st[PER];
+  float* Sg = state + ((size_t)slots[s] * I + (on ? c : 0)) * N + n0;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    a2[i] = i < nv ? A[(size_t)c * N + n0 + i] * 1.4426950408889634f : 0.f;
+    st[i] = i < nv ? Sg[i] : 0.f;
+  }
+  const float dtb = on ? dt_bias[c] : 0.f, dsk = on ? Dskip[c] : 0.f;
+  for (int tb = t0; tb < t1; tb += kST) {
+    const int n = min(kST, t1 - tb);
+    __syncthreads();
+    for (int q = tid; q < n * N; q += 256) {
+      const int tt = q / N, i = q - tt * N;
+      Bs[q] = (float)Bm[(size_t)(tb + tt) * ldb + i];
+      Cs[q] = (float)Cm[(size_t)(tb + tt) * ldc + i];
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int tt = 0; tt < n; ++tt) {
+      const size_t t = (size_t)(tb + tt);
+      const float xv = on ? x[t * ldx + c] : 0.f;
+      const float dtv = softplus_f((on ? dt[t * lddt + c] : 0.f) + dtb);
+      const float dx = dtv * xv;
+      const float* bb = Bs + tt * N + n0;
+      const float* cc = Cs + tt * N + n0;
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        if (i < nv) {
+          st[i] = fmaf(__builtin_amdgcn_exp2f(dtv * a2[i]), st[i], dx * bb[i]);
+          acc = fmaf(st[i], cc[i], acc);
+        }
+      }
+      for (int o = J >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+      if (on && j == 0) {
+        const float zv = (float)z[t * ldz + c];
+        out[t * ldo + c] = (TA)(fmaf(dsk, xv, acc) * (zv / (1.0f + expf(-zv))));
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < PER; ++i)
+    if (i < nv) Sg[i] = st[i];
 }
 
 }  // namespace
@@ -1159,8 +1236,10 @@ size_t gai_ssd_scan_ws_floats(int T, int S, int H, int N, int DV) {
 void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const void* dt, int lddt,
                   const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu,
                   const int* slots, int S, int T, float* out, int H, int G, int N, int DV, int dtt, float* ws,
-                  hipStream_t st) {
+                  hipStream_t st, const float* fixed) {
   if (S == 0) return;
+  if (!fixed && (!dt || !dt_bias || !A_log || !D))
+    gai_launch_error(__FILE__, __LINE__, "ssd_scan: step sizes, their bias, A_log and D, or a fixed decay per head");
   if (H % G) gai_launch_error(__FILE__, __LINE__, "ssd_scan: heads must be a multiple of groups");
   if (N > kMaxDK) gai_launch_error(__FILE__, __LINE__, "ssd_scan: state size above 256");
   if (T > S) {  // some sequence brings more than one row: the column-sliced scan
@@ -1174,7 +1253,7 @@ void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const 
     const size_t lds = (size_t)(2 * kTB * (RGS * R + RGS) + kTB * (64 / RGS) + 2 * kTB) * sizeof(float);             \
     ssd_scan_cols_kernel<TA, R, RGS, MODE><<<grid, 64, lds, st>>>(x, B, C, ld, (const TA*)dt, lddt, dt_bias, A_log,  \
                                                                   D, state, cu, slots, out, H, G, N, DV, S, Pbuf,   \
-                                                                  Qbuf);                                             \
+                                                                  Qbuf, fixed);                                      \
   } while (0)
 #define GAI_SSD(TA, R, RGS)                                                                                          \
   do {                                                                                                               \
@@ -1203,9 +1282,30 @@ void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const 
   const size_t lds = (size_t)(4 * N + 2 * RG * DV) * sizeof(float);
   if (dtt)
     ssd_scan_kernel<float><<<grid, DV * RG, lds, st>>>(x, B, C, ld, (const float*)dt, lddt, dt_bias, A_log, D, state, cu,
-                                                       slots, out, H, G, N, DV);
+                                                       slots, out, H, G, N, DV, fixed);
   else
     ssd_scan_kernel<bf16><<<grid, DV * RG, lds, st>>>(x, B, C, ld, (const bf16*)dt, lddt, dt_bias, A_log, D, state, cu,
-                                                      slots, out, H, G, N, DV);
+                                                      slots, out, H, G, N, DV, fixed);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_selective_scan(const float* x, int ldx, const float* dt, int lddt, const float* dt_bias, const float* A,
+                        const void* B, int ldb, const void* C, int ldc, const float* D, const void* z, int ldz,
+                        float* state, const int* cu, const int* slots, int S, void* out, int ldo, int I, int N, int dtt,
+                        hipStream_t st) {
+  if (S == 0) return;
+  if (N < 1 || N > 256) gai_launch_error(__FILE__, __LINE__, "selective_scan: 1 <= state size <= 256");
+  int J = 1;
+  while (J * 4 < N) J <<= 1;  // up to 4 states per lane, J <= 64 lanes per channel
+  const dim3 grid((unsigned)(((size_t)I * J + 255) / 256), S);
+  const size_t lds = (size_t)2 * kST * N * sizeof(float);
+  if (dtt)
+    selective_scan_kernel<float, 4><<<grid, 256, lds, st>>>(x, ldx, dt, lddt, dt_bias, A, (const float*)B, ldb,
+                                                            (const float*)C, ldc, D, (const float*)z, ldz, state, cu,
+                                                            slots, (float*)out, ldo, I, N, J);
+  else
+    selective_scan_kernel<bf16, 4><<<grid, 256, lds, st>>>(x, ldx, dt, lddt, dt_bias, A, (const bf16*)B, ldb,
+                                                           (const bf16*)C, ldc, D, (const bf16*)z, ldz, state, cu, slots,
+                                                           (bf16*)out, ldo, I, N, J);
   GAI_LAUNCH_CHECK();
 }
