@@ -7,7 +7,7 @@
 // (cap <= 0: no cap; r1 = nullptr: no distance term; window <= 0: plain causal.) Positions enter only through the
 // distance term and the window: there is no rotation. K / V live in the engine's paged cache (16-token pages,
 // K [page, G, 16, DK], V^T [page, G, DV, 16]) in bf16 or fp32; scores, softmax weights and the P.V sums are fp32.
-// Head sizes are run-time values (DK != DV allowed, DV <= 256).
+// Head sizes are run-time values (DK != DV allowed, DV <= 512).
 //
 // Sigmoid mode (template SIG): no softmax - a visible key weighs sigmoid(scale * (q_i . k_j) + bias_h) and the weights
 // are not normalised over the keys: o_i = out_scale * sum_j sigmoid(.) v_j. Same paging, tiling and key walk; the
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(const TA* __restri
   }
 }
 
-constexpr int kMaxVChunks = 4;  // DV <= 256
+constexpr int kMaxVChunks = 8;  // DV <= 512
 
 template <typename TA, bool SIG>
 __global__ __launch_bounds__(256) void window_attention_kernel(
@@ -575,7 +575,7 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
                           int ldg, const float* sig_bias, int sig, float out_scale, int dt, hipStream_t st,
                           float* part) {
   if (T == 0 || S == 0) return;
-  if (DV > 64 * kMaxVChunks) gai_launch_error(__FILE__, __LINE__, "window_attention: value head size above 256");
+  if (DV > 64 * kMaxVChunks) gai_launch_error(__FILE__, __LINE__, "window_attention: value head size above 512");
   if (H % G) gai_launch_error(__FILE__, __LINE__, "window_attention: heads must be a multiple of kv heads");
   const int TH = T * H, grid = (TH + 3) / 4;
   const size_t lds = 4 * (size_t)(DK + 64) * sizeof(float);

@@ -188,7 +188,7 @@ def random_state(cfg: LituvikConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
 
     def norm(name):
         sd[name], sd[name + ".b"] = 1 + rn(D, std=0.1), rn(D, std=0.05)
-        sd[name + ".alpha"] = un(lo=0.3, hi=0.8).reshape(())
+        sd[name + ".alpha"] = un(1, lo=0.3, hi=0.8).reshape(())
 
     def gated(p, F_):
         sd[p + "gate"], sd[p + "up"], sd[p + "down"] = lin(F_, D) * 1.5, lin(F_, D), lin(D, F_)

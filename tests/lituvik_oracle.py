@@ -80,7 +80,7 @@ def latent_attention(h, W, p, m, eps):
         first = max(0, i - win + 1) if win > 0 else 0
         for hh in range(H):
             qn, qr = q[i, hh, :dn], rotate(q[i, hh, dn:], i, freqs, mag)
-            s = torch.stack([(qn @ kn[j, hh] + qr @ kr[j]) * m["scale"] for j in range(first, i + 1)])
+            s = (kn[first:i + 1, hh] @ qn + kr[first:i + 1] @ qr) * m["scale"]
             a = torch.softmax(s, 0)
             heads[i, hh] = (a[:, None] * v[first:i + 1, hh]).sum(0)
     return heads.reshape(T, H * dv) @ W[p + "o"].T
@@ -142,19 +142,22 @@ def gated_expert(h, W, p):
     return (silu(h @ W[p + "gate"].T) * (h @ W[p + "up"].T)) @ W[p + "down"].T
 
 
-def route(h, W, p, ml):
+def route(h, W, p, ml, gaps=None):
     """-> (chosen ids [T, top], weights [T, top]); ids >= experts are identity experts."""
     top = ml["router"]["top"]
     s = torch.softmax(h @ W[p + "router"].T, -1)
     choice = s + W[p + "correction"]
     ids = torch.topk(choice, top, dim=-1).indices
+    if gaps is not None and top < choice.shape[1]:
+        srt = torch.sort(choice, -1, descending=True).values
+        gaps.append(float((srt[:, top - 1] - srt[:, top]).min()))
     w = torch.gather(s, 1, ids)
     return ids, w / (w.sum(-1, keepdim=True) + 1e-20)
 
 
-def moe_ff(h, W, p, ml):
+def moe_ff(h, W, p, ml, gaps=None):
     E = ml["router"]["experts"]
-    ids, w = route(h, W, p, ml)
+    ids, w = route(h, W, p, ml, gaps)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for j in range(ids.shape[1]):
@@ -177,8 +180,9 @@ def layer_runs(cfg):
         [(i, 0) for i in range(b, n)]
 
 
-def forward(cfg, W, tokens, residuals=None):
-    """Logits [T, vocab] of one sequence (float64). W: checkpoint tensors as float64."""
+def forward(cfg, W, tokens, residuals=None, gaps=None):
+    """Logits [T, vocab] of one sequence (float64). W: checkpoint tensors (any float type; used as float64)."""
+    W = {k: v.to(F64) for k, v in W.items()}
     eps = float(cfg["norm"]["eps"])
     x0 = W["embed"][torch.as_tensor(tokens, dtype=torch.long)]
     x = x0.clone()
@@ -200,9 +204,124 @@ def forward(cfg, W, tokens, residuals=None):
         ml = l.get("mlp")
         if ml is not None:
             h = dyt(x, W, p + "norm2")
-            x = x + (dense_ff(h, W, p + "mlp.") if ml["kind"] == "dense" else moe_ff(h, W, p + "mlp.", ml))
+            x = x + (dense_ff(h, W, p + "mlp.") if ml["kind"] == "dense" else moe_ff(h, W, p + "mlp.", ml, gaps))
         if residuals is not None:
             residuals.append(x.clone())
     logits = dyt(x, W, "final.norm") @ W["head"].T
     cap = cfg.get("logit_softcap")
     return cap * torch.tanh(logits / cap) if cap else logits
+
+
+# ------------------------------------------------------------------------------------------ made-up models for tests
+def att(heads=3, dim=8, rot_dim=4, vdim=12, kv_rank=10, scale=0.4, window=9, base=50.0, scaling=(3.0, 24, 4.0, 1.0)):
+    m = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank, scale=scale,
+             rot=dict(base=base, dims=rot_dim))
+    if window:
+        m["mask"] = dict(size=window)
+    if scaling:
+        m["rot"]["scaling"] = dict(factor=scaling[0], original=scaling[1], fast=scaling[2], slow=scaling[3])
+    return dict(type="latent_attention", mixer=m)
+
+
+def lin(heads=3, dim=8, vdim=12, decay=(0.5, 0.9, 0.99)):
+    return dict(type="lightning", mixer=dict(heads=heads, dim=dim, vdim=vdim, decay=list(decay)))
+
+
+def ssm(inner=40, state=6, dt_rank=5, conv=3):
+    return dict(type="mamba1", mixer=dict(inner=inner, state=state, dt_rank=dt_rank, conv=conv))
+
+
+def dense(layer, ff=48):
+    return dict(layer, mlp=None if ff is None else dict(kind="dense", ff=ff))
+
+
+def moe(layer, ff=24, experts=5, identity=2, top=3, shared=20):
+    ml = dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, identity=identity, top=top))
+    if shared:
+        ml["shared"] = dict(ff=shared)
+    return dict(layer, mlp=ml)
+
+
+def make_config(layers, width=32, vocab=97, eps=1e-5, loop=None, softcap=12.0):
+    c = dict(architecture="Lituvik", vocab=vocab, width=width, norm=dict(eps=eps), layers=list(layers))
+    if loop:
+        c["loop"] = dict(start=loop[0], stop=loop[1], times=loop[2])
+    if softcap:
+        c["logit_softcap"] = softcap
+    return c
+
+
+def random_checkpoint(cfg, seed, slow_decay=False):
+    """Random weights under the checkpoint's tensor names, rounded to bfloat16 (what a stored checkpoint holds), with
+    magnitudes that make every mechanism matter: norm biases, sizeable rotated parts, corrections that change the
+    choice of experts, decays from fast to slow."""
+    g = torch.Generator().manual_seed(seed)
+    D = cfg["width"]
+
+    def rn(*s, std=1.0):
+        return (torch.randn(*s, generator=g) * std).to(torch.bfloat16).float()
+
+    def un(*s, lo=0.0, hi=1.0):
+        return (torch.rand(*s, generator=g) * (hi - lo) + lo).to(torch.bfloat16).float()
+
+    def mat(o, i, gain=1.0):
+        return rn(o, i, std=gain * i ** -0.5)
+
+    W = {"embed": rn(cfg["vocab"], D), "head": mat(cfg["vocab"], D, 3.0)}
+
+    def norm(name):
+        W[name], W[name + ".b"] = un(D, lo=0.5, hi=1.5), rn(D, std=0.2)
+        W[name + ".alpha"] = un(1, lo=0.4, hi=0.9).reshape(())
+
+    def gated(p, F_):
+        W[p + "gate"], W[p + "up"], W[p + "down"] = mat(F_, D, 2.0), mat(F_, D, 1.5), mat(D, F_)
+
+    norm("final.norm")
+    for i, l in enumerate(cfg["layers"]):
+        p, x, m = f"l{i}.", f"l{i}.mix.", l["mixer"]
+        norm(p + "norm1")
+        if l["type"] == "latent_attention":
+            H, dn, dr, dv, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+            W[x + "q"], W[x + "dkv"] = mat(H * (dn + dr), D, 2.0), mat(R + dr, D, 2.0)
+            W[x + "dkv.norm"] = un(R, lo=0.5, hi=1.5)
+            W[x + "uk"], W[x + "uv"] = mat(H * dn, R, 1.5), mat(H * dv, R)
+            W[x + "o"] = mat(D, H * dv)
+        elif l["type"] == "lightning":
+            H, dk, dv = m["heads"], m["dim"], m["vdim"]
+            W[x + "q"], W[x + "k"], W[x + "v"] = mat(H * dk, D, 1.5), mat(H * dk, D, 1.5), mat(H * dv, D, 1.5)
+            W[x + "g"], W[x + "o"] = mat(H * dv, D, 2.0), mat(D, H * dv)
+            W[x + "norm"] = un(H * dv, lo=0.5, hi=1.5)
+        else:
+            I, N, rk, K = m["inner"], m["state"], m["dt_rank"], m["conv"]
+            W[x + "in"] = mat(2 * I, D, 1.5)
+            W[x + "conv"], W[x + "conv.b"] = rn(I, K, std=0.6), rn(I, std=0.2)
+            W[x + "x"] = mat(rk + 2 * N, I, 1.5)
+            W[x + "dt"] = mat(I, rk)
+            W[x + "dt.b"] = un(I, lo=-7.0, hi=-5.0) if slow_decay else un(I, lo=-3.0, hi=0.5)
+            W[x + "A_log"] = un(I, N, lo=-2.0, hi=-1.0) if slow_decay else un(I, N, lo=-1.5, hi=1.2)
+            W[x + "D"] = rn(I)
+            W[x + "o"] = mat(D, I)
+        ml = l.get("mlp")
+        if ml is None:
+            continue
+        norm(p + "norm2")
+        if ml["kind"] == "dense":
+            W[p + "mlp.up"], W[p + "mlp.down"] = mat(ml["ff"], D, 1.5), mat(D, ml["ff"])
+        else:
+            r = ml["router"]
+            n = r["experts"] + r.get("identity", 0)
+            for e in range(r["experts"]):
+                gated(p + f"mlp.e{e}.", ml["expert"]["ff"])
+            W[p + "mlp.router"] = mat(n, D, 3.0)
+            W[p + "mlp.correction"] = rn(n, std=0.15)
+            if ml.get("shared"):
+                gated(p + "mlp.shared.", ml["shared"]["ff"])
+    return W
+
+
+def router_margin(cfg, W, tokens):
+    """Smallest gap between the last chosen and the first not chosen corrected router score over all layers and
+    positions (a test with a near-tie would rest on rounding)."""
+    gaps = []
+    forward(cfg, W, tokens, gaps=gaps)
+    return min(gaps) if gaps else 1.0

@@ -1,0 +1,596 @@
+"""Lituvik decoder: the framework (model registry -> LLMEngine -> native scheduler -> ops) against the slow float64 oracle
+in tests/lituvik_oracle.py. Small made-up configurations and random weights with sizeable norm biases, rotated parts,
+router corrections and decays from fast to slow, so that a key that is one token off, a lost state, a wrong angle, a
+missing correction, a wrong expert or a wrong page moves the logits far beyond the tolerance. CPU runs use the
+reference ops, GPU runs the HIP kernels (fp32: tight tolerance; bf16: rounding level).
+"""
+import json
+import math
+import os
+
+import pytest
+import torch
+
+from generativeaiexamples_amd import ops
+from generativeaiexamples_amd.engine import EngineConfig, LLMEngine, SamplingParams
+from generativeaiexamples_amd.models.lituvik import LituvikConfig, LituvikModel
+from generativeaiexamples_amd.models.registry import build_llm
+
+from . import lituvik_oracle as O
+
+_GPU = pytest.mark.gpu
+TARGETS = [pytest.param("cpu", torch.float32, id="cpu-fp32"),
+           pytest.param("cuda", torch.float32, id="gpu-fp32", marks=_GPU),
+           pytest.param("cuda", torch.bfloat16, id="gpu-bf16", marks=_GPU)]
+FP32_TARGETS = TARGETS[:2]
+
+
+def row_err(got, want):
+    """RMS of the difference (mean over the vocabulary taken off) over the RMS of the centred reference, per row."""
+    d = got.double() - want.double()
+    d = d - d.mean(-1, keepdim=True)
+    w = want.double() - want.double().mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / w.pow(2).mean(-1).sqrt().clamp_min(1e-9)
+
+
+def rel_err(got, want):
+    return row_err(got, want).max().item()
+
+
+def close(got, want, dtype):
+    """fp32: every row within 2e-4. bf16: rounding level - rows within 4 % on average and no row beyond 15 %; a wrong
+    mechanism is off by tens of percent on most rows."""
+    e = row_err(got, want)
+    if dtype == torch.float32:
+        return e.max().item() < 2e-4
+    return e.mean().item() < 4e-2 and e.max().item() < 0.15
+
+
+def make_engine(cfg, sd, device, dtype, max_tokens=512, max_seqs=4, graphs=None):
+    model = LituvikModel(LituvikConfig.from_json(cfg), device=device, dtype=dtype).load_state(sd)
+    from generativeaiexamples_amd.engine.tokenizer import load_tokenizer
+    graphs = (device != "cpu") if graphs is None else graphs
+    return LLMEngine(model, load_tokenizer(None, "llama3", cfg["vocab"]), EngineConfig(
+        max_num_seqs=max_seqs, num_blocks=max_tokens // ops.BLOCK, max_model_len=max_tokens, max_batched_tokens=1 << 20,
+        use_graphs=graphs, graph_batch_sizes=(1, 2, 4), decode_steps=1))
+
+
+def run_schedule(eng, prompts, schedule):
+    """schedule: list of steps, each a list of (request name, count). Returns {name: logits [len, vocab]} with every
+    position's logits; requests end when their tokens are used up."""
+    at = {n: 0 for n in prompts}
+    got = {n: [] for n in prompts}
+    for step in schedule:
+        entries, end = [], []
+        for name, count in step:
+            lo = at[name]
+            entries.append((name, prompts[name][lo:lo + count], list(range(count))))
+            at[name] = lo + count
+            if at[name] == len(prompts[name]):
+                end.append(name)
+        out = eng.replay_step(entries, end)
+        r = 0
+        for name, count in step:
+            got[name].append(out[r:r + count])
+            r += count
+    return {n: torch.cat(v) for n, v in got.items() if v}
+
+
+def tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def config_for(dtype, layers, **kw):
+    """The test's configuration. An expert choice is a discrete decision: with random weights some position always has
+    two corrected router scores closer than bf16 rounding of the router's input, and the other expert's output is a
+    different vector altogether. So bf16 runs take every expert (top = experts + identity: the same kernels, no
+    decision), and the choice itself is tested in fp32 (CPU and GPU) on prompts without a near-tie (clear_tokens)."""
+    if dtype == torch.bfloat16:
+        out = []
+        for l in layers:
+            ml = l.get("mlp")
+            if ml is not None and ml["kind"] == "moe":
+                r = dict(ml["router"])
+                r["experts"] = min(r["experts"], 8 - r["identity"])
+                r["top"] = r["experts"] + r["identity"]
+                l = dict(l, mlp=dict(ml, router=r))
+            out.append(l)
+        layers = out
+    return O.make_config(layers, **kw)
+
+
+def clear_tokens(n, cfg, sd, seed, gap=1e-4):
+    """Random tokens whose router scores have no near-tie between the last chosen and the first rejected expert."""
+    for s in range(seed, seed + 50):
+        t = tokens(n, cfg["vocab"], s)
+        if O.router_margin(cfg, sd, t) > gap:
+            return t
+    raise AssertionError("no clear-cut prompt found")
+
+
+def cuts(n, sizes):
+    out, i = [], 0
+    while n > 0:
+        c = min(n, sizes[i % len(sizes)])
+        out.append(c)
+        n -= c
+        i += 1
+    return out
+
+
+FULL = [O.dense(O.ssm()), O.moe(O.att()), O.dense(O.lin()), O.moe(O.att(heads=2, dim=6, rot_dim=6, vdim=5, kv_rank=7, window=5,
+                                                                          scaling=None), top=2, identity=1, shared=None),
+        O.dense(O.ssm(inner=24, state=9, dt_rank=2, conv=4), None)]
+
+
+# ------------------------------------------------------------------------------------------------ each mechanism alone
+@pytest.mark.parametrize("device,dtype", TARGETS)
+@pytest.mark.parametrize("layer", [
+    O.dense(O.att(), None), O.dense(O.att(heads=1, dim=4, rot_dim=2, vdim=4, kv_rank=4, window=1), None),
+    O.dense(O.att(heads=5, dim=6, rot_dim=10, vdim=3, kv_rank=21, window=0, scaling=None), None),
+    O.dense(O.att(heads=2, dim=16, rot_dim=8, vdim=16, kv_rank=16, window=40, base=10000.0, scaling=(16.0, 8, 2.0, 0.5)), None),
+    O.dense(O.att(rot_dim=0, scaling=None), None),
+    O.dense(O.lin(), None), O.dense(O.lin(heads=1, dim=4, vdim=20, decay=(1.0,)), None),
+    O.dense(O.lin(heads=4, dim=20, vdim=6, decay=(0.1, 0.7, 0.95, 0.999)), None),
+    O.dense(O.ssm(), None), O.dense(O.ssm(inner=17, state=1, dt_rank=1, conv=1), None),
+    O.dense(O.ssm(inner=12, state=37, dt_rank=9, conv=5), None), O.dense(O.ssm(inner=8, state=70, dt_rank=3, conv=2), None),
+    O.dense(O.lin(), 40), O.moe(O.lin()), O.moe(O.lin(), ff=20, experts=3, identity=0, top=1, shared=None),
+    O.moe(O.ssm(), ff=40, experts=2, identity=4, top=4, shared=8), O.moe(O.att(), ff=72, experts=7, identity=1, top=8)],
+    ids=["att", "att-1head-window1", "att-uneven-causal-plainrot", "att-window40-yarn", "att-norot",
+         "lin", "lin-1head-nodecay", "lin-4heads", "ssm", "ssm-state1-conv1", "ssm-state37-conv5", "ssm-state70",
+         "dense", "moe", "moe-top1-plain", "moe-mostly-identity", "moe-top8"])
+def test_single_mechanism(layer, device, dtype):
+    cfg = config_for(dtype, [layer], width=40)
+    sd = O.random_checkpoint(cfg, 1)
+    toks = clear_tokens(37, cfg, sd, 2)
+    want = O.forward(cfg, sd, toks)
+    eng = make_engine(cfg, sd, device, dtype)
+    got = run_schedule(eng, {"a": toks}, [[("a", len(toks))]])["a"]
+    assert close(got, want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", FP32_TARGETS)
+def test_ops_against_oracle_mechanisms(device, dtype):
+    """Single ops against the oracle's functions: the tanh norm with its residual add, the rotation table, the linear
+    attention and selective scans from states that are not zero, the corrected router and the identity experts."""
+    g = torch.Generator().manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g)  # noqa: E731
+    dev = torch.device(device)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)  # noqa: E731
+    # tanh norm: residual add of one block, a second stream, the next block's norm
+    for D in (70, 64):
+        res, y, x0, w, b = rn(5, D), rn(5, D + 3), rn(5, D), rn(D), rn(D)
+        r = res.clone().to(dev)
+        out = ops.add_dyt_f32(r, y.to(dev)[:, 3:], x0.to(dev), 0.7, w.to(dev), b.to(dev), torch.float32).cpu()
+        x = res.double() + y.double()[:, 3:] + x0.double()
+        assert torch.allclose(r.cpu().double(), x, atol=1e-6)
+        assert torch.allclose(out.double(), torch.tanh(0.7 * x) * w.double() + b.double(), atol=1e-5)
+    # element-wise activations
+    a, b2 = rn(6, 50), rn(6, 50)
+    both = torch.cat([a, b2], 1).to(dev)
+    assert torch.allclose(ops.act_mul(both[:, :50], both[:, 50:], "silu").cpu().double(), O.silu(a.double()) * b2.double(), atol=1e-5)
+    assert torch.allclose(ops.act_mul(both[:, 50:], None, "relu2").cpu().double(), torch.relu(b2.double()) ** 2, atol=1e-5)
+    assert torch.allclose(ops.act_mul(both[:, :50], None, "tanh_cap", cap=1.5).cpu().double(), 1.5 * torch.tanh(a.double() / 1.5),
+                          atol=1e-5)
+    # rotation: frequencies with and without the wavelength ramp
+    for dims, base, sc in ((8, 50.0, dict(factor=4.0, original=24, fast=4.0, slow=1.0)), (6, 10000.0, None),
+                           (32, 500000.0, dict(factor=40.0, original=4096, fast=32.0, slow=1.0))):
+        inv, mag = ops.yarn_inv_freq(dims, base, sc)
+        f, m = O.yarn_frequencies(dims, base, sc)
+        assert torch.allclose(inv.double(), torch.tensor(f, dtype=torch.float64), rtol=1e-6, atol=0) and abs(mag - m) < 1e-12
+    # linear attention with constant decays from a state that is not zero, two sequences, scattered slots
+    H, dk, dv, T = 3, 5, 7, 11
+    n = 2 * H * dk + H * dv
+    qkv, st, dec = rn(T, n + 2), rn(4, H, dk, dv), torch.tensor([0.3, 0.9, 1.0])
+    cu, slots = i32([0, 4, T]), i32([2, 0])
+    s_dev, buf = st.clone().to(dev), qkv.to(dev)
+    got = ops.linear_attention_scan(buf[:, :H * dk], buf[:, H * dk:2 * H * dk], buf[:, 2 * H * dk:n], dec.to(dev), s_dev, cu,
+                                    slots).cpu().double()
+    q3, k3 = qkv[:, :H * dk].double().reshape(T, H, dk), qkv[:, H * dk:2 * H * dk].double().reshape(T, H, dk)
+    v3 = qkv[:, 2 * H * dk:n].double().reshape(T, H, dv)
+    for (lo, hi, sl) in ((0, 4, 2), (4, T, 0)):
+        for hh in range(H):
+            S = st[sl, hh].double()
+            for t in range(lo, hi):
+                S = float(dec[hh]) * S + k3[t, hh][:, None] * v3[t, hh][None, :]
+                assert torch.allclose(got[t, hh], S.T @ q3[t, hh], atol=1e-4)
+            assert torch.allclose(s_dev[sl, hh].cpu().double(), S, atol=1e-4)
+    assert torch.equal(s_dev[1].cpu(), st[1]) and torch.equal(s_dev[3].cpu(), st[3])
+    # selective scan from a state that is not zero
+    for I, N in ((10, 6), (7, 1), (5, 37), (3, 150)):
+        T = 9
+        x, dt, dtb, A, Dk = rn(T, I), rn(T, I), rn(I) - 1, -torch.exp(rn(I, N) * 0.5), rn(I)
+        bcz, st = rn(T, 2 * N + I + 1), rn(3, I, N)
+        cu, slots = i32([0, 3, T]), i32([1, 2])
+        s_dev, bz = st.clone().to(dev), bcz.to(dev)
+        got = ops.selective_scan(x.to(dev), dt.to(dev), dtb.to(dev), A.to(dev), bz[:, :N], bz[:, N:2 * N], Dk.to(dev),
+                                 bz[:, 2 * N + 1:], s_dev, cu, slots, torch.float32).cpu().double()
+        for (lo, hi, sl) in ((0, 3, 1), (3, T, 2)):
+            S = st[sl].double()
+            for t in range(lo, hi):
+                d = O.softplus(dt[t].double() + dtb.double())
+                S = torch.exp(d[:, None] * A.double()) * S + (d * x[t].double())[:, None] * bcz[t, :N].double()[None, :]
+                y = S @ bcz[t, N:2 * N].double() + Dk.double() * x[t].double()
+                assert torch.allclose(got[t], y * O.silu(bcz[t, 2 * N + 1:].double()), atol=2e-4, rtol=2e-4), (I, N, t)
+            assert torch.allclose(s_dev[sl].cpu().double(), S, atol=2e-4, rtol=2e-4)
+        assert torch.equal(s_dev[0].cpu(), st[0])
+    # router with a correction that changes the choice but not the weights; identity experts; a shared expert
+    E, NI, k, D, F_ = 4, 2, 3, 24, 16
+    h = rn(9, D)
+    Wm = {"router": rn(E + NI, D).double(), "correction": (rn(E + NI) * 0.2).double()}
+    for e in list(range(E)) + ["shared"]:
+        pre = f"e{e}." if e != "shared" else "shared."
+        Wm[pre + "gate"], Wm[pre + "up"], Wm[pre + "down"] = rn(F_, D).double(), rn(F_, D).double(), rn(D, F_).double()
+    ml = dict(kind="moe", expert=dict(ff=F_), router=dict(experts=E, identity=NI, top=k), shared=dict(ff=F_))
+    want_ids, want_w = O.route(h.double(), Wm, "", ml)
+    plain_ids = torch.topk(torch.softmax(h.double() @ Wm["router"].T, -1), k).indices
+    assert not torch.equal(torch.sort(plain_ids, -1).values, torch.sort(want_ids, -1).values)  # the correction matters
+    logits = (h.double() @ Wm["router"].T).float().to(dev)
+    ids, wts = ops.moe_route(logits, k, renorm=True, bias=Wm["correction"].float().to(dev), eps=1e-20)
+    assert torch.equal(ids.cpu().long(), want_ids) and torch.allclose(wts.cpu().double(), want_w, atol=1e-6)
+    assert (want_ids >= E).any() and (want_ids < E).any()
+    _rows, offs, pos = ops.moe_dispatch(ids, E + NI)
+    gu = torch.stack([ops.interleave_gate_up(Wm[f"e{e}.gate"].float(), Wm[f"e{e}.up"].float()) for e in range(E)]).to(dev)
+    dn = torch.stack([Wm[f"e{e}.down"].float() for e in range(E)]).to(dev)
+    hd = h.to(dev)
+    mid = ops.moe_gemm(hd, _rows, gu, offs, 9 * k, act="swiglu")
+    y = ops.moe_gemm(mid, None, dn, offs, 9 * k)
+    shared = O.gated_expert(h.double(), Wm, "shared.").float().to(dev)
+    got = ops.moe_combine(y, pos, wts, shared, ids=ids, n_real=E, identity=hd).cpu().double()
+    assert torch.allclose(got, O.moe_ff(h.double(), Wm, "", ml), atol=1e-4, rtol=1e-4)
+
+
+# ------------------------------------------------------------------------------------ whole model, schedules, batches
+@pytest.mark.parametrize("device,dtype", TARGETS)
+def test_prefill_decode_portions(device, dtype):
+    """Whole prompt, token-by-token decoding from the first token on, and portions of 2 / 3 / 5 / 17 / 1 tokens: every
+    position's logits equal the oracle's, so they do not depend on how the prompt was cut. Windows of 9 and 5 tokens end
+    inside and at the edges of portions and pages; the looped block keeps one cache / state per pass."""
+    cfg = config_for(dtype, FULL, loop=(1, 4, 2))
+    sd = O.random_checkpoint(cfg, 3)
+    toks = clear_tokens(61, cfg, sd, 4)
+    want = O.forward(cfg, sd, toks)
+    eng = make_engine(cfg, sd, device, dtype)
+    for name, sizes in (("whole", [61]), ("decode", [1]), ("prefill+decode", [30] + [1] * 31), ("small", [2, 3, 5, 17, 1]),
+                        ("twos", [2])):
+        sched = [[(name, c)] for c in cuts(61, sizes)]
+        got = run_schedule(eng, {name: toks}, sched)[name]
+        assert close(got, want, dtype), name
+
+
+@pytest.mark.parametrize("device,dtype", TARGETS)
+def test_mixed_batches_and_reuse(device, dtype):
+    """Unequal requests in one batch (portions beside single tokens) against each alone; a pool of two state slots and
+    few pages, so slots and pages of finished requests are used again by later ones."""
+    cfg = config_for(dtype, FULL[:4], loop=(2, 4, 2))
+    sd = O.random_checkpoint(cfg, 5)
+    lens = dict(a=45, b=18, c=33, d=1, e=26)
+    prompts = {n: clear_tokens(L, cfg, sd, 10 + 50 * i) for i, (n, L) in enumerate(lens.items())}
+    want = {n: O.forward(cfg, sd, t) for n, t in prompts.items()}
+    eng = make_engine(cfg, sd, device, dtype, max_tokens=96, max_seqs=2)
+    sched = [[("a", 20), ("b", 3)], [("a", 1), ("b", 15)],          # b ends: its slot and pages go back
+             [("a", 1), ("c", 2)], [("c", 17), ("a", 5)], [("a", 1), ("c", 1)], [("a", 17), ("c", 13)],  # a, c end
+             [("d", 1), ("e", 7)], [("e", 2)], [("e", 1)], [("e", 16)]]
+    got = run_schedule(eng, prompts, sched)
+    for n in prompts:
+        assert close(got[n], want[n], dtype), n
+    assert eng.sched.num_free_blocks() == 96 // ops.BLOCK and not eng.model.pool.slot_of
+
+
+@pytest.mark.parametrize("device,dtype", TARGETS)
+def test_first_tokens_and_long_decode(device, dtype):
+    """Positions 0..4 of a sequence (zero-padded convolution, zero states, one-key attention) and 150 single-token
+    steps across many page borders, past both windows and around the rotation's slow wavelengths."""
+    cfg = config_for(dtype, [O.moe(O.att(window=33)), O.dense(O.ssm(conv=4)), O.dense(O.lin(), None),
+                             O.dense(O.att(heads=2, window=16, scaling=(8.0, 16, 8.0, 2.0)))])
+    sd = O.random_checkpoint(cfg, 7)
+    toks = clear_tokens(155, cfg, sd, 8)
+    want = O.forward(cfg, sd, toks)
+    eng = make_engine(cfg, sd, device, dtype)
+    got = run_schedule(eng, {"a": toks}, [[("a", 1)] for _ in toks])["a"]
+    assert close(got[:5], want[:5], dtype)
+    assert close(got, want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", FP32_TARGETS)
+def test_far_token_through_state(device, dtype):
+    """Slowly forgetting recurrent layers (no attention): changing four tokens 300 positions back changes the last
+    logits (oracle), and the framework follows it, through a prompt cut at odd places and single-token steps."""
+    cfg = O.make_config([O.dense(O.ssm(inner=16, state=4, dt_rank=2), None),
+                         O.dense(O.lin(heads=2, dim=4, vdim=4, decay=(0.999, 1.0)), None)], width=32, vocab=64)
+    sd = O.random_checkpoint(cfg, 9, slow_decay=True)
+    a = tokens(320, cfg["vocab"], 11)
+    b = list(a)
+    for i in (5, 6, 7, 8):
+        b[i] = (b[i] + 13) % cfg["vocab"]
+    wa, wb = O.forward(cfg, sd, a)[-1:], O.forward(cfg, sd, b)[-1:]
+    assert rel_err(wb, wa) > 2e-3  # the far tokens matter
+    eng = make_engine(cfg, sd, device, dtype)
+    sched = lambda n: [[(n, c)] for c in cuts(320, [33, 2, 64, 1, 100])]  # noqa: E731
+    got = run_schedule(eng, {"a": a, "b": b}, sched("a") + sched("b"))
+    assert rel_err(got["a"][-1:], wa) < 2e-4 and rel_err(got["b"][-1:], wb) < 2e-4
+
+
+def _window_probe(device, dtype, n_ctx, hot, portion, window, R=8, DR=4, query=-1, H=2):
+    """ops-level: latent rows of n_ctx positions through the paged cache (pages deliberately scattered). Every latent is
+    orthogonal to one probing direction except the one at position `hot`, which lies along it; the query at `query`
+    points along it with a score of about 30, so the softmax puts all its weight on the hot key when that key is
+    visible. Returns the component of that query's output along the probing direction over the hot latent's:
+    about 1 if the key was seen, about 0 if not."""
+    B = ops.BLOCK
+    dev = torch.device(device)
+    nb = (n_ctx + B - 1) // B
+    pages = list(range(nb + 3))[::-1][:nb]  # not the identity
+    kc = torch.zeros(nb + 4, 1, B, R + DR, dtype=dtype, device=dev)
+    vc = torch.zeros(nb + 4, 1, R, B, dtype=dtype, device=dev)
+    g = torch.Generator().manual_seed(0)
+    qi = query % n_ctx
+    lat = torch.randn(n_ctx, R, generator=g)
+    d = torch.randn(R, generator=g)
+    d = d / d.norm()
+    lat = lat - torch.outer(lat @ d, d)
+    lat[hot] = d * 3.0
+    rotk = torch.randn(n_ctx, DR, generator=g) * 0.1          # a small rotated part: a few units of score at most
+    dkv = torch.cat([lat, rotk], 1)
+    inv, mag = ops.yarn_inv_freq(DR, 100.0, None)
+    ones = torch.ones(R, device=dev)
+    q = torch.randn(n_ctx, H, R + DR, generator=g) * 0.1      # [folded plain part | part to rotate]
+    q[qi, :, :R] = d * 30.0 / math.sqrt(R)                   # unit-RMS latents have length sqrt(R)
+    bt = torch.tensor([pages], dtype=torch.int32, device=dev)
+    done, res = 0, None
+    for c in cuts(n_ctx, portion):
+        pos = torch.arange(done, done + c)
+        slots = torch.tensor([pages[p // B] * B + p % B for p in pos.tolist()], dtype=torch.int32, device=dev)
+        qcat = torch.zeros(c, H * (R + DR), dtype=dtype, device=dev)
+        qcat.view(c, H, R + DR)[:, :, :R] = q[pos][:, :, :R].to(dev, dtype)
+        # the query's own projection holds only the part to rotate (DN = 0)
+        ops.latent_kv_write(q[pos][:, :, R:].reshape(c, H * DR).to(dev, dtype), dkv[pos].to(dev, dtype), ones, inv.to(dev),
+                            mag, pos.to(dev, torch.int32), slots, qcat, kc, vc, H, 0, DR, R, 1e-12)
+        cu = torch.tensor([0, c], dtype=torch.int32, device=dev)
+        ctx = torch.tensor([done + c], dtype=torch.int32, device=dev)
+        out = ops.window_attention(qcat, kc, vc, bt, cu, ctx, H, 1, R + DR, R, 1.0, 0.0, window)
+        if done <= qi < done + c:
+            res = out[qi - done].float().cpu().view(H, R)
+        done += c
+    return (res @ d / math.sqrt(R)).tolist()
+
+
+@pytest.mark.parametrize("device,dtype", FP32_TARGETS)
+@pytest.mark.parametrize("portion", [[1000], [1], [7, 2, 30]], ids=["prompt", "decode", "portions"])
+def test_window_edges_far_keys_and_page_borders(device, dtype, portion):
+    """One key among hundreds carries the output: the oldest key inside the window and the first outside it, keys at
+    page borders, at the first position, the query's own position (seen) and the one after it (not seen); in prompts,
+    in portions and in single-token steps."""
+    n, win = 340, 75
+    por = portion if portion != [1] else [300, 1]
+    for hot, seen in ((n - win, True), (n - win - 1, False), (n - win + 1, True), (n - 1, True), (n - 2, True), (0, False),
+                      (n - 64, True), (n - 65, True), (271, True), (272, True), (255, False), (256, False)):
+        out = _window_probe(device, dtype, n, hot, por, win)
+        assert all(abs(o - (1.0 if seen else 0.0)) < 2e-3 for o in out), (hot, seen, out)
+    for hot in (0, 1, 15, 16, 17, 31, 32, 200, n - 1):                      # no window: every earlier key is seen
+        out = _window_probe(device, dtype, n, hot, por, 0)
+        assert all(abs(o - 1.0) < 2e-3 for o in out), (hot, out)
+    for qi in (0, 5, 15, 16, 40):   # causal edge inside a portion: own position in, next position out
+        p = portion if portion != [1] else [1]
+        assert all(abs(o - 1.0) < 2e-3 for o in _window_probe(device, dtype, 70, qi, p, 20, query=qi)), qi
+        assert all(abs(o) < 2e-3 for o in _window_probe(device, dtype, 70, qi + 1, p, 20, query=qi)), qi
+    for qi, w in ((40, 8), (33, 2), (47, 16), (20, 1)):                    # window edge in the middle of a context
+        assert all(abs(o - 1.0) < 2e-3 for o in _window_probe(device, dtype, 70, qi - w + 1, p, w, query=qi)), (qi, w)
+        if w > 1:
+            assert all(abs(o) < 2e-3 for o in _window_probe(device, dtype, 70, qi - w, p, w, query=qi)), (qi, w)
+
+
+@_GPU
+@pytest.mark.parametrize("R,DR", [(64, 64), (128, 128), (96, 32), (48, 16)])
+def test_window_edges_bf16_kernels(R, DR):
+    """The same stand-out key probes in bf16: latent sizes that take the query-tiled matrix-core kernel for portions of 8
+    rows and more (key row 128 / value row 64, 256 / 128 stays on the row kernel), beside sizes off its grid."""
+    n, win, dt = 340, 75, torch.bfloat16
+    for portion in ([1000], [170, 140, 9, 11], [220, 3, 107], [329, 1]):
+        for hot, seen in ((n - win, True), (n - win - 1, False), (n - 1, True), (0, False), (n - 64, True), (256, False)):
+            out = _window_probe("cuda", dt, n, hot, portion, win, R, DR)
+            assert all(abs(o - (1.0 if seen else 0.0)) < 0.05 for o in out), (portion, hot, out)
+        for qi in (31, 32, 100):
+            assert all(abs(o - 1.0) < 0.05 for o in _window_probe("cuda", dt, 150, qi, portion, 40, R, DR, query=qi)), qi
+            assert all(abs(o) < 0.05 for o in _window_probe("cuda", dt, 150, qi + 1, portion, 40, R, DR, query=qi)), qi
+            assert all(abs(o) < 0.05 for o in _window_probe("cuda", dt, 150, qi - 40, portion, 40, R, DR, query=qi)), qi
+
+
+@_GPU
+def test_matrix_core_attention_in_model():
+    """bf16 model whose cached rows are 128 / 64 wide: portions of 8+ rows take the matrix-core attention kernel,
+    shorter ones and decoded tokens the row kernel; both against the oracle, alone and in a mixed batch."""
+    layers = [O.moe(O.att(heads=4, dim=32, rot_dim=64, vdim=32, kv_rank=64, window=48, scale=0.12, base=10000.0,
+                          scaling=(4.0, 64, 16.0, 1.0))), O.dense(O.lin(heads=2, dim=64, vdim=64, decay=(0.9, 0.99))),
+              O.dense(O.ssm(inner=256, state=16, dt_rank=8)),
+              O.dense(O.att(heads=2, dim=64, rot_dim=32, vdim=64, kv_rank=96, window=0, scale=0.1))]
+    cfg = config_for(torch.bfloat16, layers, width=128, vocab=128)
+    sd = O.random_checkpoint(cfg, 61)
+    prompts = {"a": clear_tokens(150, cfg, sd, 62), "b": clear_tokens(90, cfg, sd, 163)}
+    want = {n: O.forward(cfg, sd, t) for n, t in prompts.items()}
+    eng = make_engine(cfg, sd, "cuda", torch.bfloat16)
+    sched = [[("a", 70)], [("a", 33), ("b", 50)], [("a", 9), ("b", 1)], [("a", 1), ("b", 39)], [("a", 37)]]
+    got = run_schedule(eng, prompts, sched)
+    for n in prompts:
+        assert close(got[n], want[n], torch.bfloat16), n
+
+
+# ------------------------------------------------------------------------------------------- shapes of other models
+@pytest.mark.parametrize("device,dtype", TARGETS)
+@pytest.mark.parametrize("case", ["no-loop-no-cap", "loop-once-tail", "three-passes-middle", "tiny-odd", "wide-odd"])
+def test_other_shapes(case, device, dtype):
+    if case == "no-loop-no-cap":
+        cfg = config_for(dtype, [O.moe(O.ssm(), top=1), O.dense(O.att(window=0), None), O.dense(O.lin())], width=24, eps=1e-3,
+                         softcap=None)
+    elif case == "loop-once-tail":
+        cfg = config_for(dtype, [O.dense(O.att()), O.moe(O.lin()), O.dense(O.ssm())], loop=(0, 2, 1), width=16, vocab=33)
+    elif case == "three-passes-middle":
+        cfg = config_for(dtype, [O.dense(O.lin()), O.moe(O.att(window=4)), O.dense(O.ssm(), None), O.dense(O.lin(), None)],
+                         loop=(1, 3, 3))
+    elif case == "tiny-odd":
+        cfg = config_for(dtype, [O.moe(O.att(heads=1, dim=2, rot_dim=2, vdim=3, kv_rank=3, window=2), ff=5, experts=2, identity=1,
+                                       top=1, shared=3),
+                                 O.moe(O.ssm(inner=6, state=3, dt_rank=1, conv=2), ff=7, experts=3, identity=0, top=2, shared=None),
+                                 O.dense(O.lin(heads=1, dim=3, vdim=5, decay=(0.8,)), 9)], width=10, vocab=21, loop=(0, 3, 2))
+    else:
+        cfg = config_for(dtype, [O.moe(O.att(heads=2, dim=72, rot_dim=24, vdim=136, kv_rank=200, window=19), ff=200, experts=3,
+                                       identity=1, top=2, shared=72),
+                                 O.dense(O.ssm(inner=272, state=24, dt_rank=17), 200),
+                                 O.dense(O.lin(heads=2, dim=72, vdim=136, decay=(0.9, 0.97)), None)], width=136, vocab=150)
+    sd = O.random_checkpoint(cfg, 21)
+    toks = clear_tokens(40, cfg, sd, 22)
+    want = O.forward(cfg, sd, toks)
+    eng = make_engine(cfg, sd, device, dtype)
+    got = run_schedule(eng, {"a": toks}, [[("a", c)] for c in cuts(40, [9, 1, 1, 14])])["a"]
+    assert close(got, want, dtype)
+
+
+def test_residual_stream_after_every_layer_run():
+    """The stream after every layer run (a looped layer counts once per pass) equals the oracle's."""
+    cfg = O.make_config(FULL[:4], loop=(1, 3, 2))
+    sd = O.random_checkpoint(cfg, 71)
+    toks = clear_tokens(19, cfg, sd, 72)
+    want = []
+    O.forward(cfg, sd, toks, residuals=want)
+    eng = make_engine(cfg, sd, "cpu", torch.float32)
+    eng.model.capture_residuals = got = []
+    run_schedule(eng, {"a": toks}, [[("a", len(toks))]])
+    assert len(got) == len(want) == 6
+    for g, w in zip(got, want):
+        assert torch.allclose(g.double(), w, atol=1e-4, rtol=1e-4)
+
+
+# ------------------------------------------------------------------------------- registry, generation, runner script
+def _save(tmp_path, cfg, sd, name):
+    from safetensors.torch import save_file
+
+    d = tmp_path / name
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in sd.items()}, str(d / "model.safetensors"))
+    return d
+
+
+@pytest.mark.parametrize("device,dtype", TARGETS)
+def test_greedy_generation_through_engine(tmp_path, device, dtype):
+    """A checkpoint directory -> model registry -> LLMEngine.generate (its own scheduler, chunked prefill, decode graphs on
+    the GPU): greedy tokens equal the oracle's argmax (up to a near-tie of the oracle's top two logits)."""
+    cfg = config_for(dtype, FULL[:4], loop=(1, 3, 2))
+    sd = O.random_checkpoint(cfg, 31)
+    d = _save(tmp_path, cfg, sd, "ckpt")
+    model, tok, _ = build_llm(weights=str(d), device=device, dtype=dtype)
+    assert isinstance(model, LituvikModel) and model.dtype == dtype
+    eng = LLMEngine(model, tok, EngineConfig(max_num_seqs=4, num_blocks=64, max_model_len=256, prefill_chunk=16,
+                                             max_batched_tokens=24, graph_batch_sizes=(1, 2, 4), decode_steps=1))
+    prompts = [tokens(n, cfg["vocab"], 40 + n) for n in (23, 5, 41)]
+    reqs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    margin = 1e-3 if dtype == torch.float32 else 0.15
+    for p, r in zip(prompts, reqs):
+        assert len(r.output_ids) == 12
+        seq = list(p)
+        for t in r.output_ids:
+            row = O.forward(cfg, sd, seq)[-1]
+            assert row[t] >= row.max() - margin * (row.max() - row.min()), (len(seq), t, int(row.argmax()))
+            seq.append(t)
+
+
+def test_presets_generate():
+    """The preset of the registry runs through the engine's own entry point."""
+    model, tok, name = build_llm("tiny-lituvik", device="cpu", dtype=torch.float32)
+    assert isinstance(model, LituvikModel) and name == "tiny-lituvik"
+    eng = LLMEngine(model, tok, EngineConfig(max_num_seqs=2, num_blocks=32, max_model_len=128, use_graphs=False))
+    reqs = eng.generate([[5, 6, 7, 8, 9], [11]], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))
+    assert all(len(r.output_ids) == 6 for r in reqs)
+
+
+def test_trace_runner_script(tmp_path):
+    """bin/trace_run on the CPU: steps from stdin, logits files and 'done' lines out."""
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    cfg = O.make_config([O.moe(O.att()), O.dense(O.ssm()), O.dense(O.lin(), None)], loop=(0, 2, 2))
+    sd = O.random_checkpoint(cfg, 51)
+    d = _save(tmp_path, cfg, sd, "m")
+    a, b = clear_tokens(20, cfg, sd, 1), clear_tokens(9, cfg, sd, 102)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:12], "want": [0, 11]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[:8], "want": []}, {"id": "a", "tokens": a[12:13], "want": [0]}],
+              "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[13:], "want": [6]}, {"id": "b", "tokens": b[8:], "want": [0]}],
+              "end": ["a", "b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(d), "--dtype", "float32",
+                        "--out", str(tmp_path / "out"), "--max-tokens", "128", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    wa, wb = O.forward(cfg, sd, a), O.forward(cfg, sd, b)
+    rd = lambda n: torch.from_numpy(np.fromfile(tmp_path / "out" / f"{n}.f32", dtype="<f4").reshape(-1, cfg["vocab"]))  # noqa: E731
+    assert rel_err(rd(0), wa[[0, 11]]) < 2e-4
+    assert rel_err(rd(1), wa[[12]]) < 2e-4
+    assert rel_err(rd(2), torch.stack([wa[19], wb[8]])) < 2e-4
+
+
+def test_config_rejects_unknown_branches():
+    with pytest.raises(ValueError):
+        LituvikConfig.from_json(O.make_config([{"type": "mystery", "mixer": {}, "mlp": None}]))
+    with pytest.raises(ValueError):
+        LituvikConfig.from_json(O.make_config([dict(O.lin(), mlp={"kind": "mystery", "ff": 8})]))
+    with pytest.raises(ValueError):
+        LituvikConfig.from_json(O.make_config([O.dense(O.lin(heads=3, decay=(0.5, 0.6)))]))
+    with pytest.raises(ValueError):
+        LituvikConfig.from_json(O.make_config([O.moe(O.ssm(), experts=2, identity=1, top=4)]))
+    with pytest.raises(ValueError):
+        LituvikConfig.from_json(O.make_config([O.dense(O.att(rot_dim=3))]))
+    with pytest.raises(ValueError):
+        LituvikConfig.from_json(O.make_config([O.dense(O.lin())], loop=(0, 2, 2)))
+
+
+@_GPU
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_kernel_shape_variants(dtype):
+    """Kernel variants that the small models above do not reach - long portions of few sequences on the chunk-parallel
+    form of the scan, wide state sizes of the selective scan, the grouped expert GEMMs on and off the matrix-core grid -
+    against the same ops on the CPU (which the tests above tie to the oracle)."""
+    g = torch.Generator().manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g)  # noqa: E731
+    lim = 5e-5 if dtype == torch.float32 else 2e-2
+    rel = lambda a, b: ((a.float().cpu() - b.float()).norm() / b.float().norm()).item()  # noqa: E731
+    # linear attention: several chunks, a single token between them, a state that does not start at zero
+    for (H, N, DV) in ((4, 32, 32), (2, 100, 24), (2, 128, 128)):
+        T = 1300
+        cu = torch.tensor([0, 600, 601, 1300], dtype=torch.int32)
+        slots = torch.tensor([1, 3, 0], dtype=torch.int32)
+        qkv, st = rn(T, 2 * H * N + H * DV) * 0.3, rn(4, H, N, DV) * 0.3
+        dec = torch.linspace(0.9, 1.0, H)
+        s1, s2, qg = st.clone(), st.clone().cuda(), qkv.cuda()
+        o1 = ops.linear_attention_scan(qkv[:, :H * N], qkv[:, H * N:2 * H * N], qkv[:, 2 * H * N:], dec, s1, cu, slots)
+        o2 = ops.linear_attention_scan(qg[:, :H * N], qg[:, H * N:2 * H * N], qg[:, 2 * H * N:], dec.cuda(), s2, cu.cuda(),
+                                       slots.cuda())
+        assert rel(o2, o1) < 1e-4 and rel(s2, s1) < 1e-4, (H, N, DV)
+    # selective scan: every lane split of the state, channels off the workgroup grid, portions and single tokens
+    for (I, N) in ((300, 16), (70, 4), (33, 64), (20, 200), (513, 24)):
+        T = 150
+        cu = torch.tensor([0, 100, 101, 150], dtype=torch.int32)
+        slots = torch.tensor([2, 0, 1], dtype=torch.int32)
+        x, dt, dtb, A, Dk = rn(T, I), rn(T, I), rn(I) - 1, -torch.exp(rn(I, N) * 0.5), rn(I)
+        bcz, st = rn(T, 2 * N + I).to(dtype), rn(3, I, N)
+        s1, s2, bg = st.clone(), st.clone().cuda(), bcz.cuda()
+        o1 = ops.selective_scan(x, dt, dtb, A, bcz[:, :N], bcz[:, N:2 * N], Dk, bcz[:, 2 * N:], s1, cu, slots, dtype)
+        o2 = ops.selective_scan(x.cuda(), dt.cuda(), dtb.cuda(), A.cuda(), bg[:, :N], bg[:, N:2 * N], Dk.cuda(), bg[:, 2 * N:],
+                                s2, cu.cuda(), slots.cuda(), dtype)
+        assert rel(o2, o1) < lim and rel(s2, s1) < 1e-4, (I, N)
+    # grouped gated expert GEMMs with identity groups at the end of the offsets
+    for (D, F_) in ((128, 64), (40, 48)):
+        E, NI, k, T = 3, 2, 2, 50
+        h = rn(T, D).to(dtype)
+        gu = torch.stack([ops.interleave_gate_up(rn(F_, D) * D ** -0.5, rn(F_, D) * D ** -0.5) for _ in range(E)]).to(dtype)
+        ids = torch.randint(0, E + NI, (T, k), generator=g).int()
+        r1, offs1, _ = ops.moe_dispatch(ids, E + NI)
+        r2, offs2, _ = ops.moe_dispatch(ids.cuda(), E + NI)
+        m1 = ops.moe_gemm(h, r1, gu, offs1, T * k, act="swiglu")
+        m2 = ops.moe_gemm(h.cuda(), r2, gu.cuda(), offs2, T * k, act="swiglu")
+        nreal = int(offs1[E])
+        assert rel(m2[:nreal], m1[:nreal]) < lim, (D, F_)
