@@ -293,12 +293,12 @@ def random_checkpoint(cfg, seed, slow_decay=False):
             W[x + "norm"] = un(H * dv, lo=0.5, hi=1.5)
         else:
             I, N, rk, K = m["inner"], m["state"], m["dt_rank"], m["conv"]
-            W[x + "in"] = mat(2 * I, D, 1.5)
+            W[x + "in"] = mat(2 * I, D)
             W[x + "conv"], W[x + "conv.b"] = rn(I, K, std=0.6), rn(I, std=0.2)
-            W[x + "x"] = mat(rk + 2 * N, I, 1.5)
+            W[x + "x"] = mat(rk + 2 * N, I)
             W[x + "dt"] = mat(I, rk)
             W[x + "dt.b"] = un(I, lo=-7.0, hi=-5.0) if slow_decay else un(I, lo=-3.0, hi=0.5)
-            W[x + "A_log"] = un(I, N, lo=-2.0, hi=-1.0) if slow_decay else un(I, N, lo=-1.5, hi=1.2)
+            W[x + "A_log"] = un(I, N, lo=-2.0, hi=-1.0) if slow_decay else un(I, N, lo=-1.5, hi=0.7)
             W[x + "D"] = rn(I)
             W[x + "o"] = mat(D, I)
         ml = l.get("mlp")
