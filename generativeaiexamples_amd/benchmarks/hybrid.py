@@ -1,8 +1,10 @@
 """Prefill and decode throughput of the hybrid decoders at layer sizes of real models (random weights), side by side:
-Ronavik (sigmoid attention beside a gated linear recurrence, state-space scan layers, sigmoid-routed experts, fp32
+Lituvik (latent attention over a one-row-per-token cache, constant-decay linear attention, selective state-space scan,
+tanh norms, routed experts on the attention layers; fp32 residual / state), Ronavik (sigmoid attention beside a gated linear recurrence, state-space scan layers, sigmoid-routed experts, fp32
 post-norm residual / state), Pinavik (windowed attention + WKV + channel-decay delta rule, fp32 residual / state) and
 Qwen3-Next (gated full attention + gated DeltaNet), built at the same width, depth, head geometry and active
-feed-forward size (Ronavik: 8 experts of half the dense size, 2 per token; the others dense). `bench.py --hybrid` runs
+feed-forward size (Ronavik, and Lituvik's attention layers: 8 experts of half the dense size, 2 per token; the others
+dense). `bench.py --hybrid` runs
 it; the default workload of bench.py is untouched.
 
 Both models run through the serving engine (native scheduler, paged KV, state slots, decode graphs):
@@ -24,9 +26,10 @@ SIZES = {  # name: (width, layers, ff, heads, head_dim)
 
 def add_args(ap):
     ap.add_argument("--hybrid", action="store_true",
-                    help="prefill / decode throughput of Ronavik, Pinavik and Qwen3-Next at equal layer sizes (one GPU)")
+                    help="prefill / decode throughput of Lituvik, Ronavik, Pinavik and Qwen3-Next at equal layer sizes "
+                         "(one GPU)")
     ap.add_argument("--hybrid-sizes", default="1k,2k", help="comma list of " + ",".join(SIZES))
-    ap.add_argument("--hybrid-models", default="ronavik,pinavik,qwen3-next")
+    ap.add_argument("--hybrid-models", default="lituvik,ronavik,pinavik,qwen3-next")
     ap.add_argument("--hybrid-prefill", default="2048,8192", help="prompt lengths of the prefill measurement")
     ap.add_argument("--hybrid-decode", default="1,16,64", help="batch sizes of the decode measurement")
     ap.add_argument("--hybrid-context", type=int, default=1024)
@@ -35,6 +38,11 @@ def add_args(ap):
 
 def build(model: str, size: str, window: int, device):
     W, L, F, H, hd = SIZES[size]
+    if model == "lituvik":
+        from ..models.lituvik import LituvikConfig, LituvikModel
+
+        cfg = LituvikConfig.sized(W, L, F, H, hd, window=window, experts=8, top=2)
+        return LituvikModel(cfg, device=device).random_init(0)
     if model == "ronavik":
         from ..models.ronavik import RonavikConfig, RonavikModel
 

@@ -590,6 +590,8 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
     skip_len = kMfmaMinLen;                                                                                          \
   }
     GAI_WIN(64, 64) GAI_WIN(64, 128) GAI_WIN(128, 64) GAI_WIN(128, 128) GAI_WIN(256, 256)
+    // latent rows: key row = latent + rotated part, value row = latent
+    GAI_WIN(96, 64) GAI_WIN(192, 128) GAI_WIN(320, 256)
 #undef GAI_WIN
     GAI_LAUNCH_CHECK();
   }

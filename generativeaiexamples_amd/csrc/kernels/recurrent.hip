@@ -990,70 +990,141 @@ __global__ __launch_bounds__(256) void ssd_chunk_carry_kernel(const float* __res
 
 // ---- selective state-space scan: a decay per channel and state element ----------------------------------------------
 // Every (channel, state element) pair is its own scalar recurrence, so there is nothing to contract but the N states of
-// a channel at the output: J = 2^k lanes share a channel, each keeping up to PER states in registers (J * PER >= N), and
-// the output sum is a J-lane butterfly. B_t and C_t (shared by all channels) are staged through LDS kST tokens at a
-// time; exp(dt A) runs on the exponent unit with A pre-multiplied by log2(e). The same kernel serves prompt portions and
-// single decoded tokens (a sequence of one row).
+// a channel at the output: J = 2^k lanes share a channel, each keeping up to 4 states in registers (4 J >= N), and the
+// output sum is a J-lane butterfly. One wave64 per (64 / J channels, sequence); tokens go through in tiles of kST:
+//   A  the tile's step sizes, inputs and gates - fetched into registers one tile ahead, so their latency hides behind
+//      the serial part - become softplus(dt + bias), dt * x in LDS (token-parallel: no lane repeats another's softplus),
+//      B_t and C_t (shared by all channels) go to LDS too;
+//   B  the serial part: per token one LDS broadcast of (dt, dt x), per state exp2 (A pre-multiplied by log2 e), two
+//      FMAs, the butterfly; the channel's sum lands in LDS;
+//   C  token-parallel epilogue: (sum + D x) * silu(z), stored with the lanes along the channels.
+// The same kernel serves prompt portions and single decoded tokens (a sequence of one row).
 constexpr int kST = 16;
+constexpr int kSelPer = 4;   // states per lane
+constexpr int kSelBC = 8;    // B / C tile elements a lane prefetches (state sizes up to 32); larger states load in place
 
-template <typename TA, int PER>
-__global__ __launch_bounds__(256) void selective_scan_kernel(
+template <typename TA, int J>
+__global__ __launch_bounds__(64) void selective_scan_kernel(
     const float* __restrict__ x, int ldx, const float* __restrict__ dt, int lddt, const float* __restrict__ dt_bias,
     const float* __restrict__ A, const TA* __restrict__ Bm, int ldb, const TA* __restrict__ Cm, int ldc,
     const float* __restrict__ Dskip, const TA* __restrict__ z, int ldz, float* __restrict__ state,
-    const int* __restrict__ cu, const int* __restrict__ slots, TA* __restrict__ out, int ldo, int I, int N, int J) {
-  extern __shared__ float lds[];  // B[kST][N] | C[kST][N]
-  const int s = blockIdx.y, tid = threadIdx.x;
+    const int* __restrict__ cu, const int* __restrict__ slots, TA* __restrict__ out, int ldo, int I, int N) {
+  constexpr int CH = 64 / J, NE = kST * CH, NQ = (NE + 63) / 64;
+  extern __shared__ float lds[];  // B[kST][N] | C[kST][N] | dt[NE] | dt x[NE] | y[NE]
+  const int s = blockIdx.y, lane = threadIdx.x;
   const int t0 = cu[s], t1 = cu[s + 1];
-  if (t1 <= t0) return;  // uniform over the workgroup
+  if (t1 <= t0) return;
   float* Bs = lds;
-  float* Cs = lds + kST * N;
-  const int c = blockIdx.x * (256 / J) + tid / J, j = tid % J;
+  float* Cs = Bs + kST * N;
+  float* dtS = Cs + kST * N;
+  float* dxS = dtS + NE;
+  float* yS = dxS + NE;
+  const int c0 = blockIdx.x * CH, cl = lane / J, j = lane % J, c = c0 + cl;
   const bool on = c < I;
   const int per = (N + J - 1) / J, n0 = j * per;
   const int nv = on ? max(0, min(per, N - n0)) : 0;
-  float a2[PER], st[PER];
+  float a2[kSelPer], st[kSelPer];
   float* Sg = state + ((size_t)slots[s] * I + (on ? c : 0)) * N + n0;
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
+  for (int i = 0; i < kSelPer; ++i) {
     a2[i] = i < nv ? A[(size_t)c * N + n0 + i] * 1.4426950408889634f : 0.f;
     st[i] = i < nv ? Sg[i] : 0.f;
   }
-  const float dtb = on ? dt_bias[c] : 0.f, dsk = on ? Dskip[c] : 0.f;
+  // the tile elements (token, channel) this lane stages and finishes: e = lane + 64 q -> (e / CH, e % CH)
+  float bq[NQ], dq[NQ], rdt[NQ], rx[NQ], rz[NQ], cx[NQ], cz[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    const int ch = c0 + (lane + 64 * q) % CH;
+    bq[q] = ch < I ? dt_bias[ch] : 0.f;
+    dq[q] = ch < I ? Dskip[ch] : 0.f;
+  }
+  const bool bc_regs = kST * N <= 64 * kSelBC;
+  float rb[kSelBC], rc[kSelBC];
+  auto fetch = [&](int tb) {
+    const int n = min(kST, t1 - tb);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int e = lane + 64 * q, tt = e / CH, ch = c0 + e % CH;
+      const bool ok = e < NE && tt < n && ch < I;
+      const size_t t = (size_t)(tb + tt);
+      rdt[q] = ok ? dt[t * lddt + ch] : 0.f;
+      rx[q] = ok ? x[t * ldx + ch] : 0.f;
+      rz[q] = ok ? (float)z[t * ldz + ch] : 0.f;
+    }
+    if (bc_regs) {
+#pragma unroll
+      for (int q = 0; q < kSelBC; ++q) {
+        const int e = lane + 64 * q, tt = e / N, i = e - tt * N;
+        const bool ok = e < kST * N && tt < n;
+        rb[q] = ok ? (float)Bm[(size_t)(tb + tt) * ldb + i] : 0.f;
+        rc[q] = ok ? (float)Cm[(size_t)(tb + tt) * ldc + i] : 0.f;
+      }
+    }
+  };
+  fetch(t0);
   for (int tb = t0; tb < t1; tb += kST) {
     const int n = min(kST, t1 - tb);
-    __syncthreads();
-    for (int q = tid; q < n * N; q += 256) {
-      const int tt = q / N, i = q - tt * N;
-      Bs[q] = (float)Bm[(size_t)(tb + tt) * ldb + i];
-      Cs[q] = (float)Cm[(size_t)(tb + tt) * ldc + i];
+    // ---- A: registers -> LDS
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int e = lane + 64 * q;
+      if (e < NE) {
+        const float dtv = softplus_f(rdt[q] + bq[q]);
+        dtS[e] = dtv;
+        dxS[e] = dtv * rx[q];
+      }
+      cx[q] = rx[q];
+      cz[q] = rz[q];
+    }
+    if (bc_regs) {
+#pragma unroll
+      for (int q = 0; q < kSelBC; ++q) {
+        const int e = lane + 64 * q;
+        if (e < kST * N) {
+          Bs[e] = rb[q];
+          Cs[e] = rc[q];
+        }
+      }
+    } else {
+      for (int e = lane; e < n * N; e += 64) {
+        const int tt = e / N, i = e - tt * N;
+        Bs[e] = (float)Bm[(size_t)(tb + tt) * ldb + i];
+        Cs[e] = (float)Cm[(size_t)(tb + tt) * ldc + i];
+      }
     }
     __syncthreads();
-#pragma unroll 4
+    if (tb + kST < t1) fetch(tb + kST);  // in flight during the serial part
+    // ---- B: the recurrence
     for (int tt = 0; tt < n; ++tt) {
-      const size_t t = (size_t)(tb + tt);
-      const float xv = on ? x[t * ldx + c] : 0.f;
-      const float dtv = softplus_f((on ? dt[t * lddt + c] : 0.f) + dtb);
-      const float dx = dtv * xv;
+      const float dtv = dtS[tt * CH + cl], dx = dxS[tt * CH + cl];
       const float* bb = Bs + tt * N + n0;
       const float* cc = Cs + tt * N + n0;
       float acc = 0.f;
 #pragma unroll
-      for (int i = 0; i < PER; ++i) {
+      for (int i = 0; i < kSelPer; ++i) {
         if (i < nv) {
           st[i] = fmaf(__builtin_amdgcn_exp2f(dtv * a2[i]), st[i], dx * bb[i]);
           acc = fmaf(st[i], cc[i], acc);
         }
       }
+#pragma unroll
       for (int o = J >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-      if (on && j == 0) {
-        const float zv = (float)z[t * ldz + c];
-        out[t * ldo + c] = (TA)(fmaf(dsk, xv, acc) * (zv / (1.0f + expf(-zv))));
+      if (j == 0) yS[tt * CH + cl] = acc;
+    }
+    __syncthreads();
+    // ---- C: skip term, gate, store
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int e = lane + 64 * q, tt = e / CH, ch = c0 + e % CH;
+      if (e < NE && tt < n && ch < I) {
+        const float zv = cz[q];
+        out[(size_t)(tb + tt) * ldo + ch] = (TA)(fmaf(dq[q], cx[q], yS[e]) * (zv / (1.0f + expf(-zv))));
       }
     }
+    __syncthreads();
   }
 #pragma unroll
-  for (int i = 0; i < PER; ++i)
+  for (int i = 0; i < kSelPer; ++i)
     if (i < nv) Sg[i] = st[i];
 }
 
@@ -1296,16 +1367,25 @@ void gai_selective_scan(const float* x, int ldx, const float* dt, int lddt, cons
   if (S == 0) return;
   if (N < 1 || N > 256) gai_launch_error(__FILE__, __LINE__, "selective_scan: 1 <= state size <= 256");
   int J = 1;
-  while (J * 4 < N) J <<= 1;  // up to 4 states per lane, J <= 64 lanes per channel
-  const dim3 grid((unsigned)(((size_t)I * J + 255) / 256), S);
-  const size_t lds = (size_t)2 * kST * N * sizeof(float);
-  if (dtt)
-    selective_scan_kernel<float, 4><<<grid, 256, lds, st>>>(x, ldx, dt, lddt, dt_bias, A, (const float*)B, ldb,
-                                                            (const float*)C, ldc, D, (const float*)z, ldz, state, cu,
-                                                            slots, (float*)out, ldo, I, N, J);
-  else
-    selective_scan_kernel<bf16, 4><<<grid, 256, lds, st>>>(x, ldx, dt, lddt, dt_bias, A, (const bf16*)B, ldb,
-                                                           (const bf16*)C, ldc, D, (const bf16*)z, ldz, state, cu, slots,
-                                                           (bf16*)out, ldo, I, N, J);
+  while (J * kSelPer < N) J <<= 1;  // up to 4 states per lane, J <= 64 lanes per channel
+  const int CH = 64 / J;
+  const dim3 grid((unsigned)((I + CH - 1) / CH), S);
+  const size_t lds = (size_t)(2 * kST * N + 3 * kST * CH) * sizeof(float);
+#define GAI_SEL(TA, J_)                                                                                               \
+  selective_scan_kernel<TA, J_><<<grid, 64, lds, st>>>(x, ldx, dt, lddt, dt_bias, A, (const TA*)B, ldb, (const TA*)C, \
+                                                       ldc, D, (const TA*)z, ldz, state, cu, slots, (TA*)out, ldo, I, N)
+#define GAI_SEL_J(TA)                                                                                                 \
+  switch (J) {                                                                                                        \
+    case 1: GAI_SEL(TA, 1); break;                                                                                    \
+    case 2: GAI_SEL(TA, 2); break;                                                                                    \
+    case 4: GAI_SEL(TA, 4); break;                                                                                    \
+    case 8: GAI_SEL(TA, 8); break;                                                                                    \
+    case 16: GAI_SEL(TA, 16); break;                                                                                  \
+    case 32: GAI_SEL(TA, 32); break;                                                                                  \
+    default: GAI_SEL(TA, 64); break;                                                                                  \
+  }
+  if (dtt) { GAI_SEL_J(float) } else { GAI_SEL_J(bf16) }
+#undef GAI_SEL_J
+#undef GAI_SEL
   GAI_LAUNCH_CHECK();
 }

@@ -383,10 +383,10 @@ def test_window_edges_far_keys_and_page_borders(device, dtype, portion):
 
 
 @_GPU
-@pytest.mark.parametrize("R,DR", [(64, 64), (128, 128), (96, 32), (48, 16)])
+@pytest.mark.parametrize("R,DR", [(64, 64), (64, 32), (128, 64), (256, 64), (128, 128), (48, 16)])
 def test_window_edges_bf16_kernels(R, DR):
     """The same stand-out key probes in bf16: latent sizes that take the query-tiled matrix-core kernel for portions of 8
-    rows and more (key row 128 / value row 64, 256 / 128 stays on the row kernel), beside sizes off its grid."""
+    rows and more (key row / value row 128 / 64, 96 / 64, 192 / 128, 320 / 256), beside sizes off its grid (row kernel)."""
     n, win, dt = 340, 75, torch.bfloat16
     for portion in ([1000], [170, 140, 9, 11], [220, 3, 107], [329, 1]):
         for hot, seen in ((n - win, True), (n - win - 1, False), (n - 1, True), (0, False), (n - 64, True), (256, False)):
