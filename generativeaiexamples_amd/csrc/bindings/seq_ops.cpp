@@ -201,9 +201,9 @@ void window_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
     TORCH_CHECK(gate->size(0) == T && gate->size(1) == H * DV, "window_attention: gate shape");
   }
   float* partp = nullptr;
-  if (part) {  // scratch of the key-split decode form of the sigmoid mode
-    TORCH_CHECK(sigmoid && part->is_cuda() && part->scalar_type() == at::kFloat && part->is_contiguous() &&
-                    part->numel() >= (int64_t)gai_sigmoid_attention_splits(T, S, H) * T * H * DV,
+  if (part) {  // scratch of the key-split decode form (softmax mode keeps a maximum and a denominator per row too)
+    TORCH_CHECK(part->is_cuda() && part->scalar_type() == at::kFloat && part->is_contiguous() &&
+                    part->numel() >= (int64_t)gai_sigmoid_attention_splits(T, S, H) * T * H * (sigmoid ? DV : DV + 2),
                 "window_attention: split scratch too small");
     partp = part->data_ptr<float>();
   }
@@ -475,7 +475,7 @@ void selective_scan(const Tensor& x, const Tensor& dt, const Tensor& dt_bias, co
               "selective_scan: shapes");
   gai_selective_scan(x.data_ptr<float>(), ldx, dt.data_ptr<float>(), lddt, f32(dt_bias, "dt_bias"), f32(A, "A"),
                      B.data_ptr(), row_stride(B, "B"), C.data_ptr(), row_stride(C, "C"), f32(D, "D"), z.data_ptr(),
-                     row_stride(z, "z"), f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, out.data_ptr(), I,
+                     row_stride(z, "z"), f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, T, out.data_ptr(), I,
                      I, N, dtt, cur_stream());
 }
 

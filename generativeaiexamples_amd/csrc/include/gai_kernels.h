@@ -267,8 +267,8 @@ void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const 
 // decay per channel and state element; x / dt fp32, B / C / z / out bf16 (dtt 0) or fp32 (dtt 1)
 void gai_selective_scan(const float* x, int ldx, const float* dt, int lddt, const float* dt_bias, const float* A,
                         const void* B, int ldb, const void* C, int ldc, const float* D, const void* z, int ldz,
-                        float* state, const int* cu, const int* slots, int S, void* out, int ldo, int I, int N, int dtt,
-                        hipStream_t st);
+                        float* state, const int* cu, const int* slots, int S, int T, void* out, int ldo, int I, int N,
+                        int dtt, hipStream_t st);
 // scratch (fp32 elements) for the chunk-parallel form of a step with long portions of few sequences; 0: not chunked
 size_t gai_ssd_scan_ws_floats(int T, int S, int H, int N, int DV);
 void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,

@@ -262,10 +262,11 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
   float m = -INFINITY, l = 0.f, acc[kMaxVChunks];
 #pragma unroll
   for (int n = 0; n < kMaxVChunks; ++n) acc[n] = 0.f;
-  // sigmoid mode, decode steps: the key blocks of a row are dealt out to nsplit waves (blockIdx.y) whose unnormalised
-  // partial sums are added up by sigmoid_split_reduce_kernel - there is no softmax state to merge
+  // decode steps: the key blocks of a row are dealt out to nsplit waves (blockIdx.y). Sigmoid mode: their unnormalised
+  // partial sums are added up by sigmoid_split_reduce_kernel (no softmax state to merge); softmax mode: every split
+  // leaves (sums, running maximum, denominator) and softmax_split_reduce_kernel merges them
   int kb0 = first & ~15, kb1 = pos;
-  if (SIG && nsplit > 1) {
+  if (nsplit > 1) {
     const int nblk = (pos - kb0) / 64 + 1, per = (nblk + nsplit - 1) / nsplit;
     kb0 += (int)blockIdx.y * per * 64;
     kb1 = min(pos, kb0 + per * 64 - 1);
@@ -307,12 +308,16 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
       }
     }
   }
-  if (SIG && nsplit > 1) {
-    float* po = part + ((size_t)blockIdx.y * TH + th) * DV;
+  if (nsplit > 1) {
+    float* po = part + ((size_t)blockIdx.y * TH + th) * (SIG ? DV : DV + 2);
 #pragma unroll
     for (int n = 0; n < kMaxVChunks; ++n) {
       const int c = lane + 64 * n;
       if (c < DV) po[c] = acc[n];
+    }
+    if (!SIG && lane == 0) {
+      po[DV] = m;
+      po[DV + 1] = l;
     }
     return;
   }
@@ -339,6 +344,29 @@ __global__ __launch_bounds__(256) void sigmoid_split_reduce_kernel(const float* 
   float a = 0.f;
   for (int sp = 0; sp < nsplit; ++sp) a += part[(size_t)sp * T * HDV + e];
   out[(size_t)t * ldo + c] = (TA)(a * out_scale);
+}
+
+// out = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s (a split without keys has m = -inf, l = 0)
+template <typename TA>
+__global__ __launch_bounds__(256) void softmax_split_reduce_kernel(const float* __restrict__ part, int nsplit,
+                                                                   TA* __restrict__ out, int ldo, int T, int H, int DV,
+                                                                   const TA* __restrict__ gate, int ldg) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long)T * H * DV) return;
+  const int th = (int)(e / DV), c = (int)(e % DV), t = th / H, h = th - t * H;
+  const size_t TH = (size_t)T * H, W = DV + 2;
+  float M = -INFINITY;
+  for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, part[((size_t)sp * TH + th) * W + DV]);
+  float num = 0.f, den = 0.f;
+  for (int sp = 0; sp < nsplit; ++sp) {
+    const float* p = part + ((size_t)sp * TH + th) * W;
+    const float f = expf(p[DV] - M);
+    num = fmaf(p[c], f, num);
+    den = fmaf(p[DV + 1], f, den);
+  }
+  float y = num / den;
+  if (gate) y *= 1.0f / (1.0f + expf(-(float)gate[(size_t)t * ldg + (size_t)h * DV + c]));
+  out[(size_t)t * ldo + (size_t)h * DV + c] = (TA)y;
 }
 
 // ---- prompt portions in bf16: query tiles on the matrix cores ------------------------------------------------------
@@ -562,7 +590,7 @@ void gai_latent_kv_write(const void* q, int ldq, const void* dkv, int ldk, const
   GAI_LAUNCH_CHECK();
 }
 
-// Key splits of a sigmoid-mode decode step (every row a single token): enough waves to give each SIMD a few
+// Key splits of a decode step (every row a single token): enough waves to give each SIMD a few
 int gai_sigmoid_attention_splits(int T, int S, int H) {
   if (T != S || T * H >= 2048) return 1;
   int n = 4096 / (T * H);
@@ -595,7 +623,7 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
 #undef GAI_WIN
     GAI_LAUNCH_CHECK();
   }
-  const int nsplit = (sig && part) ? gai_sigmoid_attention_splits(T, S, H) : 1;
+  const int nsplit = part ? gai_sigmoid_attention_splits(T, S, H) : 1;
 #define GAI_ROW(TA, SIG_)                                                                                            \
   window_attention_kernel<TA, SIG_><<<dim3(grid, nsplit), 256, lds, st>>>(                                           \
       (const TA*)q, (const TA*)k_cache, (const TA*)v_cache, block_tables, maxb, cu_q, ctx, S, (TA*)out, ldo, TH, H, G, \
@@ -606,7 +634,15 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
     if (sig) GAI_ROW(bf16, true); else GAI_ROW(bf16, false);
   }
 #undef GAI_ROW
-  if (nsplit > 1) {
+  if (nsplit > 1 && !sig) {
+    const long n = (long)T * H * DV;
+    if (dt)
+      softmax_split_reduce_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(part, nsplit, (float*)out, ldo, T, H,
+                                                                                       DV, (const float*)gate, ldg);
+    else
+      softmax_split_reduce_kernel<bf16><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(part, nsplit, (bf16*)out, ldo, T, H,
+                                                                                      DV, (const bf16*)gate, ldg);
+  } else if (nsplit > 1) {
     const long n = (long)T * H * DV;
     if (dt)
       sigmoid_split_reduce_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(part, nsplit, (float*)out, ldo, T,

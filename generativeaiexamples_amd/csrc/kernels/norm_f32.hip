@@ -80,6 +80,39 @@ __global__ __launch_bounds__(256) void poly_norm_kernel(const TA* __restrict__ z
   }
 }
 
+// few wide rows (a whole-row norm in a decode step): one workgroup per (token, head), values kept in registers
+template <typename TA>
+__global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(const float* __restrict__ o, const TA* __restrict__ gate,
+                                                                  int ldg, const float* __restrict__ nw, int nw_per_head,
+                                                                  int act, TA* __restrict__ y, int H, int DV, float eps) {
+  constexpr int kMax = 32;  // DV <= 8192
+  __shared__ float scratch[16];
+  const int th = blockIdx.x, t = th / H, h = th % H, tid = threadIdx.x;
+  const float* orow = o + (size_t)th * DV;
+  float v[kMax];
+  float s = 0.f;
+#pragma unroll
+  for (int q = 0; q < kMax; ++q) {
+    const int i = tid + 256 * q;
+    v[q] = i < DV ? orow[i] : 0.f;
+    s += v[q] * v[q];
+  }
+  s = block_sum(s, scratch);
+  const float inv = 1.0f / sqrtf(s / DV + eps);
+  const TA* g = gate + (size_t)t * ldg + (size_t)h * DV;
+  const float* wr = nw + (nw_per_head ? (size_t)h * DV : 0);
+  TA* yr = y + (size_t)th * DV;
+#pragma unroll
+  for (int q = 0; q < kMax; ++q) {
+    const int i = tid + 256 * q;
+    if (i < DV) {
+      const float gv = (float)g[i];
+      const float sg = 1.0f / (1.0f + expf(-gv));
+      yr[i] = (TA)(v[q] * inv * wr[i] * (act == 0 ? gv * sg : sg));
+    }
+  }
+}
+
 template <typename TA>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const TA* __restrict__ gate,
                                                              int ldg, const float* __restrict__ nw, int nw_per_head,
@@ -325,19 +358,30 @@ __global__ __launch_bounds__(256) void add_dyt_f32_kernel(float* __restrict__ re
   for (int i = 0; i < VEC; ++i) o[i] = (TA)fmaf(tanhf(alpha * v[i]), w[c0 + i], b[c0 + i]);
 }
 
-template <typename TI, typename TO>
+template <typename TI, typename TO, int VEC>
 __global__ __launch_bounds__(256) void act_mul_kernel(const TI* __restrict__ a, int lda, const TI* __restrict__ b, int ldb,
                                                       TO* __restrict__ out, int T, int C, int act, float cap) {
+  const int per = C / VEC;
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= (long)T * C) return;
-  const int row = (int)(e / C), c = (int)(e % C);
-  const float x = (float)a[(size_t)row * lda + c];
-  float y;
-  if (act == 0) y = x / (1.0f + expf(-x));
-  else if (act == 1) y = fmaxf(x, 0.f) * fmaxf(x, 0.f);
-  else y = cap * tanhf(x / cap);
-  if (b) y *= (float)b[(size_t)row * ldb + c];
-  out[e] = (TO)y;
+  if (e >= (long)T * per) return;
+  const int row = (int)(e / per), c = (int)(e % per) * VEC;
+  struct alignas(sizeof(TI) * VEC) VI { TI v[VEC]; };
+  struct alignas(sizeof(TO) * VEC) VO { TO v[VEC]; };
+  const VI xa = *reinterpret_cast<const VI*>(a + (size_t)row * lda + c);
+  VI xb;
+  if (b) xb = *reinterpret_cast<const VI*>(b + (size_t)row * ldb + c);
+  VO yo;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    const float x = (float)xa.v[i];
+    float y;
+    if (act == 0) y = x / (1.0f + expf(-x));
+    else if (act == 1) y = fmaxf(x, 0.f) * fmaxf(x, 0.f);
+    else y = cap * tanhf(x / cap);
+    if (b) y *= (float)xb.v[i];
+    yo.v[i] = (TO)y;
+  }
+  *reinterpret_cast<VO*>(out + (size_t)row * C + c) = yo;
 }
 
 }  // namespace
@@ -369,6 +413,16 @@ void gai_head_norm_gate(const float* o, const void* gate, int ldg, const float* 
                         int T, int H, int DV, float eps, int dt, hipStream_t st) {
   if (T == 0) return;
   const int TH = T * H, grid = (TH + 3) / 4;
+  if (TH <= 256 && DV >= 1024 && DV <= 8192) {  // few wide rows: a single wave per row would walk it alone
+    if (dt)
+      head_norm_gate_wide_kernel<float><<<TH, 256, 0, st>>>(o, (const float*)gate, ldg, nw, nw_per_head, act, (float*)y,
+                                                            H, DV, eps);
+    else
+      head_norm_gate_wide_kernel<bf16><<<TH, 256, 0, st>>>(o, (const bf16*)gate, ldg, nw, nw_per_head, act, (bf16*)y, H,
+                                                           DV, eps);
+    GAI_LAUNCH_CHECK();
+    return;
+  }
   if (dt)
     head_norm_gate_kernel<float><<<grid, 256, 0, st>>>(o, (const float*)gate, ldg, nw, nw_per_head, act, (float*)y, TH,
                                                         H, DV, eps);
@@ -457,10 +511,17 @@ void gai_act_mul(const void* a, int lda, const void* b, int ldb, void* out, int 
   if (T == 0 || C == 0) return;
   if (act < 0 || act > 2) gai_launch_error(__FILE__, __LINE__, "act_mul: act 0 (silu), 1 (squared ReLU) or 2 (tanh cap)");
   if (act == 2 && !(cap > 0.f)) gai_launch_error(__FILE__, __LINE__, "act_mul: the tanh cap must be positive");
-  const long n = (long)T * C;
+  // four elements per thread where rows, strides and base addresses allow aligned vector accesses
+  const size_t esz = dt_in ? 4 : 2;
+  const bool v4 = C % 4 == 0 && lda % 4 == 0 && (!b || ldb % 4 == 0) && (uintptr_t)a % (4 * esz) == 0 &&
+                  (!b || (uintptr_t)b % (4 * esz) == 0) && (uintptr_t)out % 16 == 0;
+  const long n = (long)T * (v4 ? C / 4 : C);
   const unsigned grid = (unsigned)((n + 255) / 256);
-#define GAI_AM(TI, TO) \
-  act_mul_kernel<TI, TO><<<grid, 256, 0, st>>>((const TI*)a, lda, (const TI*)b, ldb, (TO*)out, T, C, act, cap)
+#define GAI_AM(TI, TO)                                                                                                \
+  do {                                                                                                                \
+    if (v4) act_mul_kernel<TI, TO, 4><<<grid, 256, 0, st>>>((const TI*)a, lda, (const TI*)b, ldb, (TO*)out, T, C, act, cap); \
+    else act_mul_kernel<TI, TO, 1><<<grid, 256, 0, st>>>((const TI*)a, lda, (const TI*)b, ldb, (TO*)out, T, C, act, cap);    \
+  } while (0)
   if (dt_in && dt_out) GAI_AM(float, float);
   else if (dt_in) GAI_AM(float, bf16);
   else if (dt_out) GAI_AM(bf16, float);

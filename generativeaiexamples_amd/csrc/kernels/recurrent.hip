@@ -298,6 +298,18 @@ __device__ __forceinline__ float rowgroup_sum(float v) {
   return v;
 }
 
+// Sum over J = 2^k neighbouring lanes (aligned groups), in every lane: DPP inside a row of 16, the crossbar beyond it.
+template <int J>
+__device__ __forceinline__ float lanegroup_sum(float v) {
+  if (J >= 2) v += dpp_f<0xB1>(v);
+  if (J >= 4) v += dpp_f<0x4E>(v);
+  if (J >= 8) v += dpp_f<0x141>(v);
+  if (J >= 16) v += dpp_f<0x140>(v);
+  if (J >= 32) v += __shfl_xor(v, 16, 64);
+  if (J >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
 // decay of every (token, head, channel) ahead of the serial scan: exp(-exp(wpre + w0)), token-parallel
 __global__ __launch_bounds__(256) void wkv_decay_kernel(const float* __restrict__ wpre, const float* __restrict__ w0,
                                                         float* __restrict__ wdecay, size_t n, int HD) {
@@ -990,8 +1002,10 @@ __global__ __launch_bounds__(256) void ssd_chunk_carry_kernel(const float* __res
 
 // ---- selective state-space scan: a decay per channel and state element ----------------------------------------------
 // Every (channel, state element) pair is its own scalar recurrence, so there is nothing to contract but the N states of
-// a channel at the output: J = 2^k lanes share a channel, each keeping up to 4 states in registers (4 J >= N), and the
-// output sum is a J-lane butterfly. One wave64 per (64 / J channels, sequence); tokens go through in tiles of kST:
+// a channel at the output: J = 2^k lanes share a channel, each keeping PER states in registers (PER J >= N), and the
+// output sum is a J-lane butterfly. One wave64 per (64 / J channels, sequence). PER = 4 streams the state with the fewest
+// lanes (decode steps, many sequences); PER = 1 gives a long portion of few sequences four times the waves, each with a
+// quarter of the serial work per token. Tokens go through in tiles of kST:
 //   A  the tile's step sizes, inputs and gates - fetched into registers one tile ahead, so their latency hides behind
 //      the serial part - become softplus(dt + bias), dt * x in LDS (token-parallel: no lane repeats another's softplus),
 //      B_t and C_t (shared by all channels) go to LDS too;
@@ -1000,38 +1014,41 @@ __global__ __launch_bounds__(256) void ssd_chunk_carry_kernel(const float* __res
 //   C  token-parallel epilogue: (sum + D x) * silu(z), stored with the lanes along the channels.
 // The same kernel serves prompt portions and single decoded tokens (a sequence of one row).
 constexpr int kST = 16;
-constexpr int kSelPer = 4;   // states per lane
 constexpr int kSelBC = 8;    // B / C tile elements a lane prefetches (state sizes up to 32); larger states load in place
 
-template <typename TA, int J>
+template <typename TA, int J, int PER>
 __global__ __launch_bounds__(64) void selective_scan_kernel(
     const float* __restrict__ x, int ldx, const float* __restrict__ dt, int lddt, const float* __restrict__ dt_bias,
     const float* __restrict__ A, const TA* __restrict__ Bm, int ldb, const TA* __restrict__ Cm, int ldc,
     const float* __restrict__ Dskip, const TA* __restrict__ z, int ldz, float* __restrict__ state,
     const int* __restrict__ cu, const int* __restrict__ slots, TA* __restrict__ out, int ldo, int I, int N) {
-  constexpr int CH = 64 / J, NE = kST * CH, NQ = (NE + 63) / 64;
-  extern __shared__ float lds[];  // B[kST][N] | C[kST][N] | dt[NE] | dt x[NE] | y[NE]
+  constexpr int CH = 64 / J, NE = kST * CH, NQ = (NE + 63) / 64, NP = PER * J;
+  extern __shared__ float lds[];  // B[kST][NP] | C[kST][NP] | dt[NE] | dt x[NE] | y[NE]; NP >= N, the padding stays 0
   const int s = blockIdx.y, lane = threadIdx.x;
   const int t0 = cu[s], t1 = cu[s + 1];
   if (t1 <= t0) return;
   float* Bs = lds;
-  float* Cs = Bs + kST * N;
-  float* dtS = Cs + kST * N;
+  float* Cs = Bs + kST * NP;
+  float* dtS = Cs + kST * NP;
+  for (int e = lane; e < 2 * kST * NP; e += 64) lds[e] = 0.f;
+  __syncthreads();
   float* dxS = dtS + NE;
   float* yS = dxS + NE;
   const int c0 = blockIdx.x * CH, cl = lane / J, j = lane % J, c = c0 + cl;
   const bool on = c < I;
-  const int per = (N + J - 1) / J, n0 = j * per;
-  const int nv = on ? max(0, min(per, N - n0)) : 0;
-  float a2[kSelPer], st[kSelPer];
-  float* Sg = state + ((size_t)slots[s] * I + (on ? c : 0)) * N + n0;
+  // lane j of a channel owns the states j, j + J, j + 2 J, j + 3 J; those past N are padding: decay exponent 0, B = C = 0
+  // in LDS, so they stay 0 and the serial part needs no bounds
+  float a2[PER], st[PER];
+  float* Sg = state + ((size_t)slots[s] * I + (on ? c : 0)) * N;
 #pragma unroll
-  for (int i = 0; i < kSelPer; ++i) {
-    a2[i] = i < nv ? A[(size_t)c * N + n0 + i] * 1.4426950408889634f : 0.f;
-    st[i] = i < nv ? Sg[i] : 0.f;
+  for (int i = 0; i < PER; ++i) {
+    const bool ok = on && j + J * i < N;
+    a2[i] = ok ? A[(size_t)c * N + j + J * i] * 1.4426950408889634f : 0.f;
+    st[i] = ok ? Sg[j + J * i] : 0.f;
   }
   // the tile elements (token, channel) this lane stages and finishes: e = lane + 64 q -> (e / CH, e % CH)
-  float bq[NQ], dq[NQ], rdt[NQ], rx[NQ], rz[NQ], cx[NQ], cz[NQ];
+  float bq[NQ], dq[NQ], rdt[NQ], rx[NQ], cx[NQ], cz[NQ];
+  TA rz[NQ];
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
     const int ch = c0 + (lane + 64 * q) % CH;
@@ -1039,25 +1056,33 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
     dq[q] = ch < I ? Dskip[ch] : 0.f;
   }
   const bool bc_regs = kST * N <= 64 * kSelBC;
-  float rb[kSelBC], rc[kSelBC];
+  TA rb[kSelBC], rc[kSelBC];
+  int bt[kSelBC], bi[kSelBC];
+#pragma unroll
+  for (int q = 0; q < kSelBC; ++q) {
+    bt[q] = (lane + 64 * q) / N;
+    bi[q] = (lane + 64 * q) - bt[q] * N;
+  }
+  // Loads only, from clamped (always valid) addresses: nothing here waits for the data, so the next tile's inputs are
+  // in flight while the serial part of this tile runs. Rows past the portion's end repeat its last row; they are
+  // staged but never used.
   auto fetch = [&](int tb) {
-    const int n = min(kST, t1 - tb);
+    const int last = min(kST, t1 - tb) - 1;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
-      const int e = lane + 64 * q, tt = e / CH, ch = c0 + e % CH;
-      const bool ok = e < NE && tt < n && ch < I;
-      const size_t t = (size_t)(tb + tt);
-      rdt[q] = ok ? dt[t * lddt + ch] : 0.f;
-      rx[q] = ok ? x[t * ldx + ch] : 0.f;
-      rz[q] = ok ? (float)z[t * ldz + ch] : 0.f;
+      const int e = lane + 64 * q;
+      const size_t t = (size_t)(tb + min(e / CH, last));
+      const int ch = min(c0 + e % CH, I - 1);
+      rdt[q] = dt[t * lddt + ch];
+      rx[q] = x[t * ldx + ch];
+      rz[q] = z[t * ldz + ch];
     }
     if (bc_regs) {
 #pragma unroll
       for (int q = 0; q < kSelBC; ++q) {
-        const int e = lane + 64 * q, tt = e / N, i = e - tt * N;
-        const bool ok = e < kST * N && tt < n;
-        rb[q] = ok ? (float)Bm[(size_t)(tb + tt) * ldb + i] : 0.f;
-        rc[q] = ok ? (float)Cm[(size_t)(tb + tt) * ldc + i] : 0.f;
+        const size_t t = (size_t)(tb + min(bt[q], last));
+        rb[q] = Bm[t * ldb + bi[q]];
+        rc[q] = Cm[t * ldc + bi[q]];
       }
     }
   };
@@ -1074,41 +1099,39 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
         dxS[e] = dtv * rx[q];
       }
       cx[q] = rx[q];
-      cz[q] = rz[q];
+      cz[q] = (float)rz[q];
     }
     if (bc_regs) {
 #pragma unroll
       for (int q = 0; q < kSelBC; ++q) {
         const int e = lane + 64 * q;
         if (e < kST * N) {
-          Bs[e] = rb[q];
-          Cs[e] = rc[q];
+          Bs[bt[q] * NP + bi[q]] = (float)rb[q];
+          Cs[bt[q] * NP + bi[q]] = (float)rc[q];
         }
       }
     } else {
       for (int e = lane; e < n * N; e += 64) {
         const int tt = e / N, i = e - tt * N;
-        Bs[e] = (float)Bm[(size_t)(tb + tt) * ldb + i];
-        Cs[e] = (float)Cm[(size_t)(tb + tt) * ldc + i];
+        Bs[tt * NP + i] = (float)Bm[(size_t)(tb + tt) * ldb + i];
+        Cs[tt * NP + i] = (float)Cm[(size_t)(tb + tt) * ldc + i];
       }
     }
     __syncthreads();
     if (tb + kST < t1) fetch(tb + kST);  // in flight during the serial part
     // ---- B: the recurrence
+#pragma unroll 4
     for (int tt = 0; tt < n; ++tt) {
       const float dtv = dtS[tt * CH + cl], dx = dxS[tt * CH + cl];
-      const float* bb = Bs + tt * N + n0;
-      const float* cc = Cs + tt * N + n0;
+      const float* bb = Bs + tt * NP + j;
+      const float* cc = Cs + tt * NP + j;
       float acc = 0.f;
 #pragma unroll
-      for (int i = 0; i < kSelPer; ++i) {
-        if (i < nv) {
-          st[i] = fmaf(__builtin_amdgcn_exp2f(dtv * a2[i]), st[i], dx * bb[i]);
-          acc = fmaf(st[i], cc[i], acc);
-        }
+      for (int i = 0; i < PER; ++i) {
+        st[i] = fmaf(__builtin_amdgcn_exp2f(dtv * a2[i]), st[i], dx * bb[J * i]);
+        acc = fmaf(st[i], cc[J * i], acc);
       }
-#pragma unroll
-      for (int o = J >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+      acc = lanegroup_sum<J>(acc);
       if (j == 0) yS[tt * CH + cl] = acc;
     }
     __syncthreads();
@@ -1124,8 +1147,8 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
     __syncthreads();
   }
 #pragma unroll
-  for (int i = 0; i < kSelPer; ++i)
-    if (i < nv) Sg[i] = st[i];
+  for (int i = 0; i < PER; ++i)
+    if (on && j + J * i < N) Sg[j + J * i] = st[i];
 }
 
 }  // namespace
@@ -1362,29 +1385,37 @@ void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const 
 
 void gai_selective_scan(const float* x, int ldx, const float* dt, int lddt, const float* dt_bias, const float* A,
                         const void* B, int ldb, const void* C, int ldc, const float* D, const void* z, int ldz,
-                        float* state, const int* cu, const int* slots, int S, void* out, int ldo, int I, int N, int dtt,
-                        hipStream_t st) {
+                        float* state, const int* cu, const int* slots, int S, int T, void* out, int ldo, int I, int N,
+                        int dtt, hipStream_t st) {
   if (S == 0) return;
   if (N < 1 || N > 256) gai_launch_error(__FILE__, __LINE__, "selective_scan: 1 <= state size <= 256");
-  int J = 1;
-  while (J * kSelPer < N) J <<= 1;  // up to 4 states per lane, J <= 64 lanes per channel
-  const int CH = 64 / J;
+  int J4 = 1, J1 = 1;
+  while (J4 * 4 < N) J4 <<= 1;  // 4 states per lane
+  while (J1 < N) J1 <<= 1;      // 1 state per lane
+  // portions (more rows than sequences) that would leave SIMDs idle with 4 states per lane spread over 4 x the waves
+  const bool spread = T > S && N <= 64 && (long)S * ((I * J4 + 63) / 64) < 2048;
+  const int J = spread ? J1 : J4, PER = spread ? 1 : 4, CH = 64 / J;
   const dim3 grid((unsigned)((I + CH - 1) / CH), S);
-  const size_t lds = (size_t)(2 * kST * N + 3 * kST * CH) * sizeof(float);
-#define GAI_SEL(TA, J_)                                                                                               \
-  selective_scan_kernel<TA, J_><<<grid, 64, lds, st>>>(x, ldx, dt, lddt, dt_bias, A, (const TA*)B, ldb, (const TA*)C, \
-                                                       ldc, D, (const TA*)z, ldz, state, cu, slots, (TA*)out, ldo, I, N)
-#define GAI_SEL_J(TA)                                                                                                 \
+  const size_t lds = (size_t)(2 * kST * PER * J + 3 * kST * CH) * sizeof(float);
+#define GAI_SEL(TA, J_, P_)                                                                                           \
+  selective_scan_kernel<TA, J_, P_><<<grid, 64, lds, st>>>(x, ldx, dt, lddt, dt_bias, A, (const TA*)B, ldb,           \
+                                                           (const TA*)C, ldc, D, (const TA*)z, ldz, state, cu, slots, \
+                                                           (TA*)out, ldo, I, N)
+#define GAI_SEL_J(TA, P_)                                                                                             \
   switch (J) {                                                                                                        \
-    case 1: GAI_SEL(TA, 1); break;                                                                                    \
-    case 2: GAI_SEL(TA, 2); break;                                                                                    \
-    case 4: GAI_SEL(TA, 4); break;                                                                                    \
-    case 8: GAI_SEL(TA, 8); break;                                                                                    \
-    case 16: GAI_SEL(TA, 16); break;                                                                                  \
-    case 32: GAI_SEL(TA, 32); break;                                                                                  \
-    default: GAI_SEL(TA, 64); break;                                                                                  \
+    case 1: GAI_SEL(TA, 1, P_); break;                                                                                \
+    case 2: GAI_SEL(TA, 2, P_); break;                                                                                \
+    case 4: GAI_SEL(TA, 4, P_); break;                                                                                \
+    case 8: GAI_SEL(TA, 8, P_); break;                                                                                \
+    case 16: GAI_SEL(TA, 16, P_); break;                                                                              \
+    case 32: GAI_SEL(TA, 32, P_); break;                                                                              \
+    default: GAI_SEL(TA, 64, P_); break;                                                                              \
   }
-  if (dtt) { GAI_SEL_J(float) } else { GAI_SEL_J(bf16) }
+  if (dtt) {
+    if (PER == 1) { GAI_SEL_J(float, 1) } else { GAI_SEL_J(float, 4) }
+  } else {
+    if (PER == 1) { GAI_SEL_J(bf16, 1) } else { GAI_SEL_J(bf16, 4) }
+  }
 #undef GAI_SEL_J
 #undef GAI_SEL
   GAI_LAUNCH_CHECK();

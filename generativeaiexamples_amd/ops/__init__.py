@@ -1160,8 +1160,12 @@ def window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H: int, G: in
         return ref.window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H, G, DK, DV, scale, softcap, window,
                                     r1, r2, gate)
     out = torch.empty(q.shape[0], H * DV, dtype=q.dtype, device=q.device)
+    # decode steps of few rows: the keys of a row are split over several waves, merged from (sums, maximum, denominator)
+    T, S = q.shape[0], ctx.numel()
+    ns = native().sigmoid_attention_splits(T, S, H)
+    part = torch.empty(ns * T * H * (DV + 2), dtype=torch.float32, device=q.device) if ns > 1 else None
     native().window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, out, H, G, DK, DV, float(scale),
-                              float(softcap or 0.0), int(window or 0), r1, r2, gate, None, False, 1.0, None)
+                              float(softcap or 0.0), int(window or 0), r1, r2, gate, None, False, 1.0, part)
     return out
 
 
