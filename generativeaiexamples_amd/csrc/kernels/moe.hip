@@ -44,8 +44,8 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int T, int E,
     else
       for (int e = 0; e < E; ++e) s += __expf(x[e] - mx);
   }
-  float bv[8];
-  int bi[8];
+  float bv[16];
+  int bi[16];
   for (int j = 0; j < k; ++j) {
     bv[j] = -INFINITY;
     bi[j] = 0;
@@ -479,7 +479,7 @@ void gai_moe_dispatch(const int* ids, int n, int k, int E, int* a_rows, int* off
 void gai_moe_route(const float* logits, int T, int E, int k, int renorm, int* ids, float* w, hipStream_t st,
                    int sigmoid, const float* bias, float eps) {
   if (T == 0) return;
-  if (k < 1 || k > 8 || k > E) gai_launch_error(__FILE__, __LINE__, "moe_route: 1 <= top-k <= min(8, experts)");
+  if (k < 1 || k > 16 || k > E) gai_launch_error(__FILE__, __LINE__, "moe_route: 1 <= top-k <= min(16, experts)");
   moe_route_kernel<<<(T + 255) / 256, 256, 0, st>>>(logits, T, E, k, renorm, ids, w, sigmoid, bias, eps);
   GAI_LAUNCH_CHECK();
 }

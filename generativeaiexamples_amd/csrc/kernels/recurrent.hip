@@ -1009,8 +1009,9 @@ __global__ __launch_bounds__(256) void ssd_chunk_carry_kernel(const float* __res
 //   A  the tile's step sizes, inputs and gates - fetched into registers one tile ahead, so their latency hides behind
 //      the serial part - become softplus(dt + bias), dt * x in LDS (token-parallel: no lane repeats another's softplus),
 //      B_t and C_t (shared by all channels) go to LDS too;
-//   B  the serial part: per token one LDS broadcast of (dt, dt x), per state exp2 (A pre-multiplied by log2 e), two
-//      FMAs, the butterfly; the channel's sum lands in LDS;
+//   B  the serial part, a few tokens at a time: decays exp2(dt A) (A pre-multiplied by log2 e), dt x B and C of those
+//      tokens first (independent, pipelined), then one FMA per state and token on the dependency chain, then the
+//      butterflies of all those tokens; the channel's sums land in LDS;
 //   C  token-parallel epilogue: (sum + D x) * silu(z), stored with the lanes along the channels.
 // The same kernel serves prompt portions and single decoded tokens (a sequence of one row).
 constexpr int kST = 16;
@@ -1119,20 +1120,40 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
     }
     __syncthreads();
     if (tb + kST < t1) fetch(tb + kST);  // in flight during the serial part
-    // ---- B: the recurrence
-#pragma unroll 4
-    for (int tt = 0; tt < n; ++tt) {
-      const float dtv = dtS[tt * CH + cl], dx = dxS[tt * CH + cl];
-      const float* bb = Bs + tt * NP + j;
-      const float* cc = Cs + tt * NP + j;
-      float acc = 0.f;
+    // ---- B: the recurrence, SUB tokens at a time: everything off the dependency chain (decays, dt x B, C) is computed
+    // for the SUB tokens first, so the chain itself is one FMA per state and token; rows past the portion's end are
+    // staged (repeats of its last row) and made neutral here
+    constexpr int SUB = kST / PER;
+    for (int ts = 0; ts < n; ts += SUB) {
+      float dec[PER][SUB], dxb[PER][SUB], ccv[PER][SUB], accv[SUB];
 #pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        st[i] = fmaf(__builtin_amdgcn_exp2f(dtv * a2[i]), st[i], dx * bb[J * i]);
-        acc = fmaf(st[i], cc[J * i], acc);
+      for (int u = 0; u < SUB; ++u) {
+        const int tt = ts + u;
+        const bool live = tt < n;
+        const float dtv = dtS[tt * CH + cl], dx = dxS[tt * CH + cl];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          dec[i][u] = live ? __builtin_amdgcn_exp2f(dtv * a2[i]) : 1.0f;
+          dxb[i][u] = live ? dx * Bs[tt * NP + j + J * i] : 0.f;
+          ccv[i][u] = Cs[tt * NP + j + J * i];
+        }
       }
-      acc = lanegroup_sum<J>(acc);
-      if (j == 0) yS[tt * CH + cl] = acc;
+#pragma unroll
+      for (int u = 0; u < SUB; ++u) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          st[i] = fmaf(dec[i][u], st[i], dxb[i][u]);
+          acc = fmaf(st[i], ccv[i][u], acc);
+        }
+        accv[u] = acc;
+      }
+#pragma unroll
+      for (int u = 0; u < SUB; ++u) accv[u] = lanegroup_sum<J>(accv[u]);
+      if (j == 0) {
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) yS[(ts + u) * CH + cl] = accv[u];
+      }
     }
     __syncthreads();
     // ---- C: skip term, gate, store

@@ -94,8 +94,8 @@ class LituvikConfig:
                 if kind == "moe":
                     r = dict(ml["router"])
                     r.setdefault("identity", 0)
-                    if not 1 <= r["top"] <= min(8, r["experts"] + r["identity"]):
-                        raise ValueError(f"layer {i}: 1 <= top <= min(8, experts + identity)")
+                    if not 1 <= r["top"] <= min(16, r["experts"] + r["identity"]):
+                        raise ValueError(f"layer {i}: 1 <= top <= min(16, experts + identity)")
                     ml["router"] = r
             layers.append(dict(l, mixer=m, mlp=ml))
         self.layers = tuple(layers)
