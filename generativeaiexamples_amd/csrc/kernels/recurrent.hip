@@ -1172,6 +1172,67 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
     if (on && j + J * i < N) Sg[j + J * i] = st[i];
 }
 
+// Single-token steps (every sequence brings one row): no tiles to stage - a thread owns four neighbouring states of a
+// channel (one 16-byte state load and store where N % 4 == 0), J lanes a channel; the step is state-bandwidth bound.
+// Longer sequences would be walked token by token (correct, not fast): the launcher sends them to the tiled kernel.
+template <typename TA, int J>
+__global__ __launch_bounds__(256) void selective_step_kernel(
+    const float* __restrict__ x, int ldx, const float* __restrict__ dt, int lddt, const float* __restrict__ dt_bias,
+    const float* __restrict__ A, const TA* __restrict__ Bm, int ldb, const TA* __restrict__ Cm, int ldc,
+    const float* __restrict__ Dskip, const TA* __restrict__ z, int ldz, float* __restrict__ state,
+    const int* __restrict__ cu, const int* __restrict__ slots, TA* __restrict__ out, int ldo, int I, int N) {
+  const int s = blockIdx.y;
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  const int g = blockIdx.x * 256 + threadIdx.x, c = g / J, j = g % J, n0 = 4 * j;
+  const bool on = c < I;
+  float* Sg = state + ((size_t)slots[s] * I + (on ? c : 0)) * N + n0;
+  const bool vec = on && (N & 3) == 0 && n0 < N;
+  float a2[4], st[4];
+  if (vec) {
+    const float4 a = *reinterpret_cast<const float4*>(A + (size_t)c * N + n0);
+    const float4 v = *reinterpret_cast<const float4*>(Sg);
+    a2[0] = a.x, a2[1] = a.y, a2[2] = a.z, a2[3] = a.w;
+    st[0] = v.x, st[1] = v.y, st[2] = v.z, st[3] = v.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool ok = on && n0 + i < N;
+      a2[i] = ok ? A[(size_t)c * N + n0 + i] : 0.f;
+      st[i] = ok ? Sg[i] : 0.f;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a2[i] *= 1.4426950408889634f;
+  const float dtb = on ? dt_bias[c] : 0.f, dsk = on ? Dskip[c] : 0.f;
+  for (int t = t0; t < t1; ++t) {
+    const float xv = on ? x[(size_t)t * ldx + c] : 0.f;
+    const float dtv = softplus_f((on ? dt[(size_t)t * lddt + c] : 0.f) + dtb);
+    const float dx = dtv * xv;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (on && n0 + i < N) {
+        const float bv = (float)Bm[(size_t)t * ldb + n0 + i], cv = (float)Cm[(size_t)t * ldc + n0 + i];
+        st[i] = fmaf(__builtin_amdgcn_exp2f(dtv * a2[i]), st[i], dx * bv);
+        acc = fmaf(st[i], cv, acc);
+      }
+    }
+    acc = lanegroup_sum<J>(acc);
+    if (on && j == 0) {
+      const float zv = (float)z[(size_t)t * ldz + c];
+      out[(size_t)t * ldo + c] = (TA)(fmaf(dsk, xv, acc) * (zv / (1.0f + expf(-zv))));
+    }
+  }
+  if (vec) {
+    *reinterpret_cast<float4*>(Sg) = make_float4(st[0], st[1], st[2], st[3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (on && n0 + i < N) Sg[i] = st[i];
+  }
+}
+
 }  // namespace
 
 void gai_token_shift_mix(const void* h, const float* mu, int NM, const float* shift_state, const int* cu,
@@ -1413,6 +1474,27 @@ void gai_selective_scan(const float* x, int ldx, const float* dt, int lddt, cons
   int J4 = 1, J1 = 1;
   while (J4 * 4 < N) J4 <<= 1;  // 4 states per lane
   while (J1 < N) J1 <<= 1;      // 1 state per lane
+  if (T == S) {  // single-token steps
+    const dim3 sgrid((unsigned)(((size_t)I * J4 + 255) / 256), S);
+#define GAI_STEP(TA, J_)                                                                                              \
+  selective_step_kernel<TA, J_><<<sgrid, 256, 0, st>>>(x, ldx, dt, lddt, dt_bias, A, (const TA*)B, ldb, (const TA*)C, \
+                                                       ldc, D, (const TA*)z, ldz, state, cu, slots, (TA*)out, ldo, I, N)
+#define GAI_STEP_J(TA)                                                                                                \
+  switch (J4) {                                                                                                       \
+    case 1: GAI_STEP(TA, 1); break;                                                                                   \
+    case 2: GAI_STEP(TA, 2); break;                                                                                   \
+    case 4: GAI_STEP(TA, 4); break;                                                                                   \
+    case 8: GAI_STEP(TA, 8); break;                                                                                   \
+    case 16: GAI_STEP(TA, 16); break;                                                                                 \
+    case 32: GAI_STEP(TA, 32); break;                                                                                 \
+    default: GAI_STEP(TA, 64); break;                                                                                 \
+  }
+    if (dtt) { GAI_STEP_J(float) } else { GAI_STEP_J(bf16) }
+#undef GAI_STEP_J
+#undef GAI_STEP
+    GAI_LAUNCH_CHECK();
+    return;
+  }
   // portions (more rows than sequences) that would leave SIMDs idle with 4 states per lane spread over 4 x the waves
   const bool spread = T > S && N <= 64 && (long)S * ((I * J4 + 63) / 64) < 2048;
   const int J = spread ? J1 : J4, PER = spread ? 1 : 4, CH = 64 / J;
