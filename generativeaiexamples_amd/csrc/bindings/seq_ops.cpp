@@ -416,7 +416,7 @@ void latent_kv_write(const Tensor& q, const Tensor& dkv, const Tensor& nw, const
   const int ldq = row_stride(q, "q"), ldk = row_stride(dkv, "dkv");
   const int T = q.size(0);
   TORCH_CHECK(q.size(1) == H * (DN + DR) && dkv.size(0) == T && dkv.size(1) == R + DR && nw.numel() == R &&
-                  inv_freq.numel() == DR / 2 && DR % 2 == 0 && positions.numel() >= T && slots.numel() >= T &&
+                  2 * inv_freq.numel() <= DR && positions.numel() >= T && slots.numel() >= T &&
                   q_cat.is_contiguous() && q_cat.numel() == (int64_t)T * H * (R + DR),
               "latent_kv_write: shapes");
   TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() && k_cache.size(1) == 1 && k_cache.size(2) == 16 &&
@@ -424,9 +424,9 @@ void latent_kv_write(const Tensor& q, const Tensor& dkv, const Tensor& nw, const
                   v_cache.size(2) == R && v_cache.size(3) == 16 && v_cache.size(0) == k_cache.size(0),
               "latent_kv_write: cache pages K [pages, 1, 16, R + DR], V^T [pages, 1, R, 16]");
   gai_latent_kv_write(q.data_ptr(), ldq, dkv.data_ptr(), ldk, f32(nw, "norm weight"),
-                      DR ? f32(inv_freq, "inv_freq") : nullptr, (float)mag, i32(positions, "positions"),
+                      inv_freq.numel() ? f32(inv_freq, "inv_freq") : nullptr, (float)mag, i32(positions, "positions"),
                       i32(slots, "slots"), q_cat.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), T, (int)H, (int)DN,
-                      (int)DR, (int)R, (float)eps, dt, cur_stream());
+                      (int)DR, (int)R, (float)eps, dt, cur_stream(), 2 * (int)inv_freq.numel());
 }
 
 void linear_attention_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& decay, Tensor& state,

@@ -229,7 +229,7 @@ void gai_act_mul(const void* a, int lda, const void* b, int ldb, void* out, int 
                  int dt_out, hipStream_t st);
 void gai_latent_kv_write(const void* q, int ldq, const void* dkv, int ldk, const float* nw, const float* inv_freq,
                          float mag, const int* positions, const int* slots, void* q_cat, void* k_cache, void* v_cache,
-                         int T, int H, int DN, int DR, int R, float eps, int dt, hipStream_t st);
+                         int T, int H, int DN, int DR, int R, float eps, int dt, hipStream_t st, int ROT);
 // attention_window.hip
 void gai_qknorm_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* wq,
                          const float* wk, const int* slots, void* q_out, void* k_cache, void* v_cache, int T, int H,

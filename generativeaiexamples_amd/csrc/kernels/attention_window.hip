@@ -24,8 +24,8 @@
 // channels of the down projection) * w plus DR rotated key channels shared by all heads: K page row [c | kr] (one kv
 // head, key size R + DR), V^T page c. The rotated DR channels of every query head go to the tail of that head's row of
 // q_cat (whose first R channels hold the query folded through the key expansion), so window_attention scores against
-// the cached row directly. Rotation: channel i pairs with i + DR / 2, angle = position * inv_freq[i] (fp32, libm
-// sincosf), cos and sin times one magnitude.
+// the cached row directly. Rotation over the first ROT of the DR channels (the rest pass unchanged): channel i pairs
+// with i + ROT / 2, angle = position * inv_freq[i] (fp32, libm sincosf), cos and sin times one magnitude.
 //
 // window_attention, row kernel: one wave64 per (token, head) (a sequence is (cu_q[s], ctx[s]); the query at row t has
 // position ctx - q_len + (t - cu_q)). Keys are walked in page-aligned blocks of 64: lane j scores key j (q broadcast
@@ -183,10 +183,10 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(const TA* __restri
                                                               const int* __restrict__ positions,
                                                               const int* __restrict__ slots, TA* __restrict__ q_cat,
                                                               TA* __restrict__ k_cache, TA* __restrict__ v_cache, int H,
-                                                              int DN, int DR, int R, float eps) {
-  extern __shared__ float cs[];  // cos[DR / 2] | sin[DR / 2]
+                                                              int DN, int DR, int R, float eps, int ROT) {
+  extern __shared__ float cs[];  // cos[ROT / 2] | sin[ROT / 2]
   __shared__ float scratch[16];
-  const int t = blockIdx.x, tid = threadIdx.x, half = DR >> 1;
+  const int t = blockIdx.x, tid = threadIdx.x, half = ROT >> 1;
   const TA* lr = dkv + (size_t)t * ldk;
   const float pos = (float)positions[t];
   for (int i = tid; i < half; i += 256) {
@@ -216,6 +216,12 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(const TA* __restri
     const float u = (float)lr[R + i], v = (float)lr[R + half + i], c = cs[i], sn = cs[half + i];
     kr[R + i] = (TA)(u * c - v * sn);
     kr[R + half + i] = (TA)(v * c + u * sn);
+  }
+  const int rest = DR - ROT;  // channels past the rotated ones pass unchanged
+  for (int i = tid; i < rest; i += 256) kr[R + ROT + i] = lr[R + ROT + i];
+  for (int x = tid; x < H * rest; x += 256) {
+    const int h = x / rest, i = x - h * rest;
+    q_cat[((size_t)t * H + h) * DK + R + ROT + i] = q[(size_t)t * ldq + (size_t)h * (DN + DR) + DN + ROT + i];
   }
   for (int x = tid; x < H * half; x += 256) {
     const int h = x / half, i = x - h * half;
@@ -575,18 +581,19 @@ void gai_headnorm_kv_write(const void* q, int ldq, const void* k, int ldk, const
 
 void gai_latent_kv_write(const void* q, int ldq, const void* dkv, int ldk, const float* nw, const float* inv_freq,
                          float mag, const int* positions, const int* slots, void* q_cat, void* k_cache, void* v_cache,
-                         int T, int H, int DN, int DR, int R, float eps, int dt, hipStream_t st) {
+                         int T, int H, int DN, int DR, int R, float eps, int dt, hipStream_t st, int ROT) {
   if (T == 0) return;
-  if (DR % 2 || R < 1) gai_launch_error(__FILE__, __LINE__, "latent_kv_write: even rotated size, latent size >= 1");
-  const size_t lds = (size_t)(DR > 0 ? DR : 1) * sizeof(float);
+  if (ROT % 2 || ROT < 0 || ROT > DR || R < 1)
+    gai_launch_error(__FILE__, __LINE__, "latent_kv_write: an even number of rotated channels within DR, latent size >= 1");
+  const size_t lds = (size_t)(ROT > 0 ? ROT : 1) * sizeof(float);
   if (dt)
     latent_kv_write_kernel<float><<<T, 256, lds, st>>>((const float*)q, ldq, (const float*)dkv, ldk, nw, inv_freq, mag,
                                                        positions, slots, (float*)q_cat, (float*)k_cache,
-                                                       (float*)v_cache, H, DN, DR, R, eps);
+                                                       (float*)v_cache, H, DN, DR, R, eps, ROT);
   else
     latent_kv_write_kernel<bf16><<<T, 256, lds, st>>>((const bf16*)q, ldq, (const bf16*)dkv, ldk, nw, inv_freq, mag,
                                                       positions, slots, (bf16*)q_cat, (bf16*)k_cache, (bf16*)v_cache, H,
-                                                      DN, DR, R, eps);
+                                                      DN, DR, R, eps, ROT);
   GAI_LAUNCH_CHECK();
 }
 

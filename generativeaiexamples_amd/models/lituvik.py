@@ -75,8 +75,9 @@ class LituvikConfig:
                 m.setdefault("scale", (m["dim"] + m["rot_dim"]) ** -0.5)
                 rot = dict(m.get("rot") or {})
                 rot.setdefault("base", 10000.0)
-                if int(rot.setdefault("dims", m["rot_dim"])) != m["rot_dim"] or m["rot_dim"] % 2:
-                    raise ValueError(f"layer {i}: the rotation covers the rot_dim channels, an even number")
+                dims = int(rot.setdefault("dims", m["rot_dim"]))
+                if dims % 2 or not 0 <= dims <= m["rot_dim"]:
+                    raise ValueError(f"layer {i}: the rotation covers an even number of the rot_dim channels")
                 m["rot"] = rot
             elif l["type"] == "lightning":
                 m.setdefault("vdim", m["dim"])
@@ -310,8 +311,8 @@ class LituvikModel:
                 w[x + "dkv.norm"] = f32(sd[x + "dkv.norm"])
                 w[x + "uk"] = mat(sd[x + "uk"].float().reshape(H, dn, R))                     # q_plain [H, T, dn] @ this
                 w[x + "uv"] = mat(sd[x + "uv"].float().reshape(H, m["vdim"], R).transpose(1, 2))  # [H, R, dv]
-                inv, mag = ops.yarn_inv_freq(m["rot_dim"], m["rot"]["base"], m["rot"].get("scaling")) \
-                    if m["rot_dim"] else (torch.zeros(0), 1.0)
+                inv, mag = ops.yarn_inv_freq(m["rot"]["dims"], m["rot"]["base"], m["rot"].get("scaling")) \
+                    if m["rot"]["dims"] else (torch.zeros(0), 1.0)
                 self.rot[i] = (inv.to(dev), mag)
             elif l["type"] == "lightning":
                 w[x + "in"] = mat(torch.cat([sd[x + k] for k in ("q", "k", "v", "g")]))

@@ -1352,8 +1352,9 @@ def latent_kv_write(q, dkv, norm_w, inv_freq, mag: float, positions, slots, q_ca
     kr = rot(dkv[:, R:R + DR]) are the whole cache row - K page row [c | kr] (one kv head of key size R + DR), V^T
     page c - and the rotated part of every query head (q [T, H * (DN + DR)], the last DR channels of each head) lands
     in q_cat[:, h, R:] (q_cat [T, H * (R + DR)]; its first R channels per head hold the query folded through the key
-    expansion). The rotation pairs channel i with i + DR / 2 and turns by positions * inv_freq[i]; cos and sin are
-    multiplied by mag (see yarn_inv_freq). Angles, cos / sin and the norm are fp32."""
+    expansion). The rotation covers the first 2 * len(inv_freq) of the DR channels (the rest pass unchanged): it pairs
+    channel i with i + len(inv_freq) and turns by positions * inv_freq[i]; cos and sin are multiplied by mag (see
+    yarn_inv_freq). Angles, cos / sin and the norm are fp32."""
     if not q.is_cuda:
         return ref.latent_kv_write(q, dkv, norm_w, inv_freq, mag, positions, slots, q_cat, k_cache, v_cache, H, DN, DR,
                                    R, eps)

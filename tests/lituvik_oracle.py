@@ -67,7 +67,7 @@ def latent_attention(h, W, p, m, eps):
     T = h.shape[0]
     H, dn, dr, dv, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
     rot = m.get("rot") or {}
-    freqs, mag = yarn_frequencies(dr, float(rot.get("base", 10000.0)), rot.get("scaling"))
+    freqs, mag = yarn_frequencies(int(rot.get("dims", dr)), float(rot.get("base", 10000.0)), rot.get("scaling"))
     win = int((m.get("mask") or {}).get("size") or 0)
     q = (h @ W[p + "q"].T).reshape(T, H, dn + dr)
     low = h @ W[p + "dkv"].T
@@ -213,9 +213,10 @@ def forward(cfg, W, tokens, residuals=None, gaps=None):
 
 
 # ------------------------------------------------------------------------------------------ made-up models for tests
-def att(heads=3, dim=8, rot_dim=4, vdim=12, kv_rank=10, scale=0.4, window=9, base=50.0, scaling=(3.0, 24, 4.0, 1.0)):
+def att(heads=3, dim=8, rot_dim=4, vdim=12, kv_rank=10, scale=0.4, window=9, base=50.0, scaling=(3.0, 24, 4.0, 1.0),
+        dims=None):
     m = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank, scale=scale,
-             rot=dict(base=base, dims=rot_dim))
+             rot=dict(base=base, dims=rot_dim if dims is None else dims))
     if window:
         m["mask"] = dict(size=window)
     if scaling:

@@ -131,14 +131,14 @@ FULL = [O.dense(O.ssm()), O.moe(O.att()), O.dense(O.lin()), O.moe(O.att(heads=2,
     O.dense(O.att(), None), O.dense(O.att(heads=1, dim=4, rot_dim=2, vdim=4, kv_rank=4, window=1), None),
     O.dense(O.att(heads=5, dim=6, rot_dim=10, vdim=3, kv_rank=21, window=0, scaling=None), None),
     O.dense(O.att(heads=2, dim=16, rot_dim=8, vdim=16, kv_rank=16, window=40, base=10000.0, scaling=(16.0, 8, 2.0, 0.5)), None),
-    O.dense(O.att(rot_dim=0, scaling=None), None),
+    O.dense(O.att(rot_dim=0, scaling=None), None), O.dense(O.att(rot_dim=10, dims=6), None),
     O.dense(O.lin(), None), O.dense(O.lin(heads=1, dim=4, vdim=20, decay=(1.0,)), None),
     O.dense(O.lin(heads=4, dim=20, vdim=6, decay=(0.1, 0.7, 0.95, 0.999)), None),
     O.dense(O.ssm(), None), O.dense(O.ssm(inner=17, state=1, dt_rank=1, conv=1), None),
     O.dense(O.ssm(inner=12, state=37, dt_rank=9, conv=5), None), O.dense(O.ssm(inner=8, state=70, dt_rank=3, conv=2), None),
     O.dense(O.lin(), 40), O.moe(O.lin()), O.moe(O.lin(), ff=20, experts=3, identity=0, top=1, shared=None),
     O.moe(O.ssm(), ff=40, experts=2, identity=4, top=4, shared=8), O.moe(O.att(), ff=72, experts=7, identity=1, top=8)],
-    ids=["att", "att-1head-window1", "att-uneven-causal-plainrot", "att-window40-yarn", "att-norot",
+    ids=["att", "att-1head-window1", "att-uneven-causal-plainrot", "att-window40-yarn", "att-norot", "att-part-rotated",
          "lin", "lin-1head-nodecay", "lin-4heads", "ssm", "ssm-state1-conv1", "ssm-state37-conv5", "ssm-state70",
          "dense", "moe", "moe-top1-plain", "moe-mostly-identity", "moe-top8"])
 def test_single_mechanism(layer, device, dtype):
@@ -544,7 +544,7 @@ def test_config_rejects_unknown_branches():
     with pytest.raises(ValueError):
         LituvikConfig.from_json(O.make_config([O.moe(O.ssm(), experts=2, identity=1, top=4)]))
     with pytest.raises(ValueError):
-        LituvikConfig.from_json(O.make_config([O.dense(O.att(rot_dim=3))]))
+        LituvikConfig.from_json(O.make_config([O.dense(O.att(rot_dim=4, dims=3))]))
     with pytest.raises(ValueError):
         LituvikConfig.from_json(O.make_config([O.dense(O.lin())], loop=(0, 2, 2)))
 
