@@ -167,6 +167,14 @@ def test_ops_against_oracle_mechanisms(device, dtype):
         x = res.double() + y.double()[:, 3:] + x0.double()
         assert torch.allclose(r.cpu().double(), x, atol=1e-6)
         assert torch.allclose(out.double(), torch.tanh(0.7 * x) * w.double() + b.double(), atol=1e-5)
+    res, y, w, b = rn(7, 64), rn(7, 64), rn(64), rn(64)          # rows and strides that take the four-wide path
+    r = res.clone().to(dev)
+    out = ops.add_dyt_f32(r, y.to(dev), None, 1.3, w.to(dev), b.to(dev), torch.float32).cpu()
+    assert torch.allclose(out.double(), torch.tanh(1.3 * (res.double() + y.double())) * w.double() + b.double(), atol=1e-5)
+    wide = rn(6, 72).to(dev)
+    for lo in (0, 2, 4):                                          # aligned and misaligned column slices of 64
+        got = ops.act_mul(wide[:, lo:lo + 64], wide[:, 8:72], "silu").cpu().double()
+        assert torch.allclose(got, O.silu(wide[:, lo:lo + 64].cpu().double()) * wide[:, 8:72].cpu().double(), atol=1e-5), lo
     # element-wise activations
     a, b2 = rn(6, 50), rn(6, 50)
     both = torch.cat([a, b2], 1).to(dev)
