@@ -69,12 +69,13 @@ void head_norm_gate(const Tensor& o, const Tensor& gate, const Tensor& nw, int64
   const int dt = act_dt(gate, "gate");
   same_dt(y, dt, "y");
   const int ldg = row_stride(gate, "gate");
-  TORCH_CHECK(gate.size(0) == T && gate.size(1) == H * DV && y.is_contiguous() && y.numel() == o.numel(),
+  const int ldy = row_stride(y, "y");
+  TORCH_CHECK(gate.size(0) == T && gate.size(1) == H * DV && y.size(0) == T && y.size(1) == H * DV,
               "head_norm_gate: gate / y shapes");
   TORCH_CHECK(nw.numel() == DV || nw.numel() == H * DV, "head_norm_gate: norm weight size");
   TORCH_CHECK(act == 0 || act == 1, "head_norm_gate: act 0 (silu) or 1 (sigmoid)");
   gai_head_norm_gate(f32(o, "o"), gate.data_ptr(), ldg, f32(nw, "nw"), nw.numel() == H * DV && H > 1 ? 1 : 0, (int)act,
-                     y.data_ptr(), T, H, DV, (float)eps, dt, cur_stream());
+                     y.data_ptr(), ldy, T, H, DV, (float)eps, dt, cur_stream());
 }
 
 void embed_scale_f32(const Tensor& ids, const Tensor& table, double scale, Tensor& out,
@@ -96,21 +97,22 @@ void embed_scale_f32(const Tensor& ids, const Tensor& table, double scale, Tenso
                       pos_table ? pos_table->data_ptr() : nullptr, P);
 }
 
-void gated_norm_add_f32(Tensor& res, const Tensor& y, const Tensor& gate, const Tensor& wpost, double eps,
+void gated_norm_add_f32(Tensor& res, const Tensor& y, const optional<Tensor>& gate, const Tensor& wpost, double eps,
                         const optional<Tensor>& wnext, optional<Tensor> out) {
   TORCH_CHECK(res.dim() == 2, "gated_norm_add_f32: res [T, D]");
   float* r = f32w(res, "res");
   const int T = res.size(0), D = res.size(1);
-  const int dty = act_dt(y, "y"), dtg = act_dt(gate, "gate");
-  TORCH_CHECK(y.size(0) == T && y.size(1) == D && gate.size(0) == T && gate.size(1) == D && wpost.numel() == D,
-              "gated_norm_add_f32: y / gate / weight shapes");
+  const int dty = act_dt(y, "y"), dtg = gate ? act_dt(*gate, "gate") : dty;
+  TORCH_CHECK(y.size(0) == T && y.size(1) == D && (!gate || (gate->size(0) == T && gate->size(1) == D)) &&
+                  wpost.numel() == D, "gated_norm_add_f32: y / gate / weight shapes");
   int dto = 0;
   if (out) {
     dto = act_dt(*out, "out");
     TORCH_CHECK(out->is_contiguous() && out->numel() == (int64_t)T * D, "gated_norm_add_f32: out shape");
   }
   if (wnext) TORCH_CHECK(wnext->numel() == D, "gated_norm_add_f32: next norm weight size");
-  gai_gated_norm_add_f32(r, y.data_ptr(), row_stride(y, "y"), dty, gate.data_ptr(), row_stride(gate, "gate"), dtg,
+  gai_gated_norm_add_f32(r, y.data_ptr(), row_stride(y, "y"), dty, gate ? gate->data_ptr() : nullptr,
+                         gate ? row_stride(*gate, "gate") : 0, dtg,
                          f32(wpost, "wpost"), wnext ? f32(*wnext, "wnext") : nullptr, out ? out->data_ptr() : nullptr,
                          dto, T, D, (float)eps, cur_stream());
 }
@@ -179,7 +181,8 @@ void window_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
                       const Tensor& cu_q, const Tensor& ctx, Tensor& out, int64_t H, int64_t G, int64_t DK, int64_t DV,
                       double scale, double softcap, int64_t window, const optional<Tensor>& r1,
                       const optional<Tensor>& r2, const optional<Tensor>& gate, const optional<Tensor>& sig_bias,
-                      bool sigmoid, double out_scale, const optional<Tensor>& part) {
+                      bool sigmoid, double out_scale, const optional<Tensor>& part, int64_t chunk,
+                      const optional<Tensor>& head_scale, const optional<double>& sink) {
   const int dt = act_dt(q, "q");
   same_dt(out, dt, "out");
   check_cache(k_cache, v_cache, dt, G, DK, DV);
@@ -190,7 +193,8 @@ void window_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
   TORCH_CHECK(out.size(0) == T && out.size(1) == H * DV && cu_q.numel() == S + 1 && block_tables.dim() == 2 &&
                   block_tables.size(0) >= S, "window_attention: out / cu_q / block table shapes");
   if (sig_bias) TORCH_CHECK(sigmoid && sig_bias->numel() == H, "window_attention: one sigmoid bias per head");
-  TORCH_CHECK(sigmoid || out_scale == 1.0, "window_attention: an output scale needs the sigmoid mode");
+  if (head_scale) TORCH_CHECK(!sigmoid && head_scale->numel() == H, "window_attention: one score scale per head, softmax mode");
+  TORCH_CHECK(chunk >= 0 && (!sigmoid || (chunk == 0 && !sink)), "window_attention: chunks and sinks go with the softmax mode");
   if (sigmoid) TORCH_CHECK(!gate && !r1 && softcap == 0.0, "window_attention: sigmoid mode takes no cap, distance term or gate");
   TORCH_CHECK(r1.has_value() == r2.has_value(), "window_attention: r1 and r2 come together");
   if (r1) TORCH_CHECK(r1->numel() == H && r2->numel() == H, "window_attention: one distance pair per head");
@@ -212,7 +216,67 @@ void window_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
                        (float)scale, (float)softcap, (int)window, r1 ? f32(*r1, "r1") : nullptr,
                        r2 ? f32(*r2, "r2") : nullptr, gate ? gate->data_ptr() : nullptr, ldg,
                        sig_bias ? f32(*sig_bias, "sig_bias") : nullptr, sigmoid ? 1 : 0, (float)out_scale, dt,
-                       cur_stream(), partp);
+                       cur_stream(), partp, (int)chunk, head_scale ? f32(*head_scale, "head_scale") : nullptr, sink ? 1 : 0,
+                       sink ? (float)*sink : 0.f);
+}
+
+void rotary_kv_write(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& positions, const Tensor& slots,
+                     Tensor& q_out, Tensor& k_cache, Tensor& v_cache, int64_t H, int64_t G, int64_t DK, int64_t DV,
+                     int64_t rot, double base) {
+  const int di = act_dt(q, "q"), dt = act_dt(k_cache, "k_cache");
+  same_dt(k, di, "k");
+  same_dt(v, di, "v");
+  same_dt(q_out, dt, "q_out");
+  check_cache(k_cache, v_cache, dt, G, DK, DV);
+  const int T = q.size(0);
+  TORCH_CHECK(q.size(1) == H * DK && k.size(0) == T && k.size(1) == G * DK && v.size(0) == T && v.size(1) == G * DV,
+              "rotary_kv_write: projection shapes");
+  TORCH_CHECK(slots.numel() >= T && positions.numel() >= T && q_out.is_contiguous() && q_out.numel() == (int64_t)T * H * DK,
+              "rotary_kv_write: slot / position / output shapes");
+  TORCH_CHECK(di == 1 || dt == 0, "rotary_kv_write: bf16 inputs go with a bf16 cache");
+  gai_rotary_kv_write(q.data_ptr(), row_stride(q, "q"), k.data_ptr(), row_stride(k, "k"), v.data_ptr(), row_stride(v, "v"),
+                      i32(positions, "positions"), i32(slots, "slots"), q_out.data_ptr(), k_cache.data_ptr(),
+                      v_cache.data_ptr(), T, H, G, DK, DV, (int)rot, (float)base, di, dt, cur_stream());
+}
+
+void decay_gate(const Tensor& z, const optional<Tensor>& bias, int64_t kind, double param, Tensor& out) {
+  const int dt = act_dt(z, "z");
+  const int T = z.size(0), C = z.size(1);
+  TORCH_CHECK(kind >= 0 && kind <= 2 && out.numel() == (int64_t)T * C, "decay_gate: kind 0 .. 2, out [T, C]");
+  if (bias) TORCH_CHECK(bias->numel() == C, "decay_gate: one bias per channel");
+  gai_decay_gate(z.data_ptr(), row_stride(z, "z"), bias ? f32(*bias, "bias") : nullptr, (int)kind, (float)param,
+                 f32w(out, "out"), T, C, dt, cur_stream());
+}
+
+void unit_key_removal(const Tensor& k, const Tensor& a, const optional<Tensor>& a_bias, int64_t H, int64_t DK, double eps,
+                      Tensor& av, Tensor& bv) {
+  const int dt = act_dt(k, "k");
+  same_dt(a, dt, "a");
+  const int T = k.size(0);
+  TORCH_CHECK(k.size(1) == H * DK && a.size(0) == T && a.size(1) == H * DK && av.numel() == (int64_t)T * H * DK &&
+                  bv.numel() == av.numel(), "unit_key_removal: k / a [T, H * DK]");
+  if (a_bias) TORCH_CHECK(a_bias->numel() == H * DK, "unit_key_removal: one bias per channel");
+  gai_unit_key_removal(k.data_ptr(), row_stride(k, "k"), a.data_ptr(), row_stride(a, "a"),
+                       a_bias ? f32(*a_bias, "a_bias") : nullptr, f32w(av, "av"), f32w(bv, "bv"), T, H, DK, (float)eps, dt,
+                       cur_stream());
+}
+
+void dplr_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& decay, const optional<Tensor>& av,
+               const optional<Tensor>& bv, Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& out,
+               double q_scale) {
+  const int dt = act_dt(q, "q");
+  same_dt(k, dt, "k");
+  same_dt(v, dt, "v");
+  TORCH_CHECK(state.dim() == 4, "dplr_scan: state [slots, H, DK, DV]");
+  const int T = q.size(0), H = state.size(1), DK = state.size(2), DV = state.size(3), S = slots.numel();
+  TORCH_CHECK(q.size(1) == H * DK && k.size(0) == T && k.size(1) == H * DK && v.size(0) == T && v.size(1) == H * DV &&
+                  decay.numel() == (int64_t)T * H * DK && out.numel() == (int64_t)T * H * DV && cu.numel() == S + 1,
+              "dplr_scan: q / k / decay [T, H * DK], v [T, H * DV], out [T, H, DV]");
+  TORCH_CHECK(av.has_value() == bv.has_value(), "dplr_scan: the two removal vectors come together");
+  if (av) TORCH_CHECK(av->numel() == decay.numel() && bv->numel() == decay.numel(), "dplr_scan: av / bv [T, H * DK]");
+  gai_dplr_scan(q.data_ptr(), row_stride(q, "q"), k.data_ptr(), row_stride(k, "k"), v.data_ptr(), row_stride(v, "v"),
+                f32(decay, "decay"), av ? f32(*av, "av") : nullptr, bv ? f32(*bv, "bv") : nullptr, f32w(state, "state"),
+                i32(cu, "cu"), i32(slots, "slots"), S, T, f32w(out, "out"), H, DK, DV, (float)q_scale, dt, cur_stream());
 }
 
 void token_shift_mix(const Tensor& h, const Tensor& mu, const Tensor& shift_state, const Tensor& cu, const Tensor& slots,
@@ -493,6 +557,10 @@ void gai_bind_seq_ops(pybind11::module_& m) {
   m.def("embed_scale_f32", &embed_scale_f32);
   m.def("qknorm_kv_write", &qknorm_kv_write);
   m.def("window_attention", &window_attention);
+  m.def("rotary_kv_write", &rotary_kv_write);
+  m.def("decay_gate", &decay_gate);
+  m.def("unit_key_removal", &unit_key_removal);
+  m.def("dplr_scan", &dplr_scan);
   m.def("sigmoid_attention_splits", [](int64_t T, int64_t S, int64_t H) { return (int64_t)gai_sigmoid_attention_splits(T, S, H); });
   m.def("token_shift_mix", &token_shift_mix);
   m.def("state_tail_write", &state_tail_write);

@@ -498,8 +498,24 @@ void gemm_fp8(const Tensor& A, const Tensor& B, const Tensor& sa, const Tensor& 
                opt_ptr(R), M, N, K, ldc, (int)epi, f32 ? 1 : 0, (int)force, cur_stream());
 }
 
+void moe_route_grouped(const Tensor& logits, int64_t k, Tensor& ids, Tensor& w, const optional<Tensor>& bias, double eps,
+                       int64_t groups, int64_t keep, double scale) {
+  check_f32(logits, "router logits");
+  check_i32(ids, "topk ids");
+  check_f32(w, "topk weights");
+  TORCH_CHECK(logits.dim() == 2 && logits.is_contiguous() && ids.is_contiguous() && w.is_contiguous() &&
+                  ids.numel() == logits.size(0) * k && w.numel() == ids.numel(), "moe_route: logits [T, E], ids / w [T, k]");
+  if (bias) {
+    check_f32(*bias, "choice bias");
+    TORCH_CHECK(bias->is_contiguous() && bias->numel() == logits.size(1), "moe_route: bias [E]");
+  }
+  gai_moe_route_grouped(logits.data_ptr<float>(), logits.size(0), logits.size(1), (int)k, ids.data_ptr<int>(),
+                        w.data_ptr<float>(), bias ? bias->data_ptr<float>() : nullptr, (float)eps, (int)groups, (int)keep,
+                        (float)scale, cur_stream());
+}
+
 void moe_gemm(const Tensor& A, const optional<Tensor>& a_rows, const Tensor& W, Tensor& C, const Tensor& offs,
-              int64_t rows_total, int64_t act) {
+              int64_t rows_total, int64_t act, double act_param) {
   const bool f32 = A.scalar_type() == at::kFloat;
   if (f32) {
     check_f32(A, "A");
@@ -514,10 +530,11 @@ void moe_gemm(const Tensor& A, const optional<Tensor>& a_rows, const Tensor& W, 
   if (a_rows) check_i32(*a_rows, "a_rows");
   TORCH_CHECK(W.dim() == 3 && W.size(2) == A.size(-1) && W.is_contiguous() && A.is_contiguous(),
               "moe_gemm: W must be [E, N, K]");
-  TORCH_CHECK(offs.numel() >= W.size(0) + 1 && C.numel() == rows_total * (act == 1 ? W.size(1) / 2 : W.size(1)) &&
+  TORCH_CHECK(offs.numel() >= W.size(0) + 1 && C.numel() == rows_total * (act == 1 || act == 3 ? W.size(1) / 2 : W.size(1)) &&
                   (a_rows ? a_rows->numel() >= rows_total : A.size(0) >= rows_total), "moe_gemm: row / offset shapes");
   gai_moe_gemm(A.data_ptr(), a_rows ? a_rows->data_ptr<int>() : nullptr, W.data_ptr(), C.data_ptr(),
-               offs.data_ptr<int>(), W.size(0), rows_total, W.size(1), W.size(2), (int)act, cur_stream(), f32 ? 1 : 0);
+               offs.data_ptr<int>(), W.size(0), rows_total, W.size(1), W.size(2), (int)act, cur_stream(), f32 ? 1 : 0,
+               (float)act_param);
 }
 
 void moe_dispatch(const Tensor& ids, int64_t E, Tensor& a_rows, Tensor& offs, Tensor& pos) {
@@ -537,8 +554,15 @@ void moe_dispatch(const Tensor& ids, int64_t E, Tensor& a_rows, Tensor& offs, Te
 }
 
 void moe_combine(const Tensor& Y, const Tensor& pos, const optional<Tensor>& w, const optional<Tensor>& residual,
-                 Tensor& out, const optional<Tensor>& ids, int64_t n_real, const optional<Tensor>& ident) {
+                 Tensor& out, const optional<Tensor>& ids, int64_t n_real, const optional<Tensor>& ident,
+                 const optional<Tensor>& rgate) {
   const bool f32 = out.scalar_type() == at::kFloat;
+  int ldrg = 0;
+  if (rgate) {  // one logit per token: [T] or a [T, 1] column of a wider row
+    TORCH_CHECK(residual && rgate->is_cuda() && rgate->scalar_type() == out.scalar_type() && rgate->size(0) == pos.size(0) &&
+                    rgate->numel() == pos.size(0), "moe_combine: residual gate [T] in the rows' dtype, with a residual");
+    ldrg = (int)rgate->stride(0);
+  }
   TORCH_CHECK(Y.scalar_type() == out.scalar_type(), "moe_combine: Y / out dtypes differ");
   if (ids) {
     check_i32(*ids, "ids");
@@ -562,7 +586,7 @@ void moe_combine(const Tensor& Y, const Tensor& pos, const optional<Tensor>& w, 
   if (residual) TORCH_CHECK(residual->is_contiguous() && residual->numel() == out.numel(), "moe_combine: residual shape");
   gai_moe_combine(Y.data_ptr(), pos.data_ptr<int>(), w ? w->data_ptr<float>() : nullptr, opt_ptr(residual),
                   out.data_ptr(), T, k, D, cur_stream(), f32 ? 1 : 0, ids ? ids->data_ptr<int>() : nullptr, (int)n_real,
-                  ident ? ident->data_ptr() : nullptr);
+                  ident ? ident->data_ptr() : nullptr, rgate ? rgate->data_ptr() : nullptr, ldrg);
 }
 
 void embedding(const Tensor& ids, const Tensor& table, Tensor& out, int64_t vstart, int64_t vend) {
@@ -989,6 +1013,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_route", &moe_route);
   m.def("moe_scale_rows", &moe_scale_rows);
   m.def("moe_gemm", &moe_gemm);
+  m.def("moe_route_grouped", &moe_route_grouped);
   m.def("moe_combine", &moe_combine);
   m.def("moe_dispatch", &moe_dispatch);
   m.def("moe_dispatch_by", &moe_dispatch_by);

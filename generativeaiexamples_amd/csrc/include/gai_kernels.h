@@ -145,11 +145,14 @@ void gai_moe_route(const float* logits, int T, int E, int k, int renorm, int* id
                    int sigmoid = 0, const float* bias = nullptr, float eps = 0.f);
 // dt: 0 bf16 (MFMA tiles when K % 64 == 0), 1 fp32 (generic grouped kernel, true fp32)
 void gai_moe_gemm(const void* A, const int* a_rows, const void* W, void* C, const int* offs, int E, int rows_total,
-                  int N, int K, int act, hipStream_t st, int dt = 0);
+                  int N, int K, int act, hipStream_t st, int dt = 0, float actp = 0.f);
+// sigmoid scores, choice on score + bias among the experts of the KEEP best of NG groups, weights renormalised * scale
+void gai_moe_route_grouped(const float* logits, int T, int E, int k, int* ids, float* w, const float* bias, float eps,
+                           int NG, int KEEP, float scale, hipStream_t st);
 // w = nullptr: plain sum of the k rows
 void gai_moe_combine(const void* Y, const int* pos, const float* w, const void* residual, void* out, int T, int k,
                      int D, hipStream_t st, int dt = 0, const int* ids = nullptr, int n_real = 0,
-                     const void* ident = nullptr);
+                     const void* ident = nullptr, const void* rgate = nullptr, int ldrg = 0);
 void gai_moe_scale_rows(const void* h, const int* pos, const float* w, void* out, int T, int k, int D, int dt,
                         hipStream_t st);
 
@@ -213,7 +216,7 @@ void gai_add_rmsnorm_f32(float* res, const void* delta, int ldd, float mult, con
                          float eps, int dt_delta, int dt_out, hipStream_t st);
 void gai_poly_norm(const void* z, void* y, const float* coef, int T, int F, float eps, int dt, hipStream_t st);
 void gai_head_norm_gate(const float* o, const void* gate, int ldg, const float* nw, int nw_per_head, int act, void* y,
-                        int T, int H, int DV, float eps, int dt, hipStream_t st);
+                        int ldy, int T, int H, int DV, float eps, int dt, hipStream_t st);
 void gai_embed_scale_f32(const int* ids, const void* table, float scale, float* out, int T, int D, int V, int dt,
                          hipStream_t st, const int* positions = nullptr, const void* pos_table = nullptr, int P = 0);
 void gai_gated_norm_add_f32(float* res, const void* y, int ldy, int dt_y, const void* gate, int ldg, int dt_gate,
@@ -224,7 +227,7 @@ void gai_gate_group_norm(const float* y, const void* z, int ldz, const float* w,
 // res += delta (+ extra); out = tanh(alpha res) * w + b (out may be null)
 void gai_add_dyt_f32(float* res, const void* delta, int ldd, const float* extra, float alpha, const float* w,
                      const float* b, void* out, int T, int D, int dt_delta, int dt_out, hipStream_t st);
-// out = act(a) (* b): act 0 silu, 1 squared ReLU, 2 cap * tanh(a / cap)
+// out = act(a) (* b): act 0 silu, 1 squared ReLU, 2 cap * tanh(a / cap), 3 tanh GELU, 4 clamped gated (a, b; limit cap)
 void gai_act_mul(const void* a, int lda, const void* b, int ldb, void* out, int T, int C, int act, float cap, int dt_in,
                  int dt_out, hipStream_t st);
 void gai_latent_kv_write(const void* q, int ldq, const void* dkv, int ldk, const float* nw, const float* inv_freq,
@@ -243,10 +246,24 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
                           const int* cu_q, const int* ctx, int S, void* out, int ldo, int T, int H, int G, int DK, int DV,
                           float scale, float softcap, int window, const float* r1, const float* r2, const void* gate,
                           int ldg, const float* sig_bias, int sig, float out_scale, int dt, hipStream_t st,
-                          float* part = nullptr);
+                          float* part = nullptr, int chunk = 0, const float* hscale = nullptr, int has_sink = 0,
+                          float sink = 0.f);
+// q / k heads rotated in interleaved pairs over their first ROT channels; dt_in: input type, dt: cache / q_out type
+void gai_rotary_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const int* positions,
+                         const int* slots, void* q_out, void* k_cache, void* v_cache, int T, int H, int G, int DK, int DV,
+                         int ROT, float base, int dt_in, int dt, hipStream_t st);
 // sigmoid-mode decode steps: number of key splits (1: none); part must hold splits * T * H * DV floats
 int gai_sigmoid_attention_splits(int T, int S, int H);
 // recurrent.hip
+// kind 0 sigmoid(x), 1 sigmoid(x)^(1 / param), 2 exp(-param sigmoid(x)); x = z + bias
+void gai_decay_gate(const void* z, int ldz, const float* bias, int kind, float param, float* out, int T, int C, int dt,
+                    hipStream_t st);
+void gai_unit_key_removal(const void* k, int ldk, const void* a, int lda, const float* a_bias, float* av, float* bv, int T,
+                          int H, int DK, float eps, int dt, hipStream_t st);
+// S <- diag(decay) S - av (bv^T S) + k v^T (av = nullptr: no removal), o = q_scale S^T q
+void gai_dplr_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* decay,
+                   const float* av, const float* bv, float* state, const int* cu, const int* slots, int S, int T,
+                   float* out, int H, int DK, int DV, float q_scale, int dt, hipStream_t st);
 void gai_token_shift_mix(const void* h, const float* mu, int NM, const float* shift_state, const int* cu,
                          const int* slots, int S, void* out, int T, int D, int dt, hipStream_t st);
 void gai_state_tail_write(const void* x, int ldx, float* state, const int* cu, const int* slots, int S, int C, int NR,

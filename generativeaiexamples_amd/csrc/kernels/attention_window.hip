@@ -13,6 +13,15 @@
 // are not normalised over the keys: o_i = out_scale * sum_j sigmoid(.) v_j. Same paging, tiling and key walk; the
 // running maximum, the rescaling of the accumulators and the final division drop out.
 //
+// Chunk mode (chunk > 0): a key is visible only inside the query's own chunk of positions, floor(j / chunk) ==
+// floor(i / chunk), counted from position 0 of the sequence. hscale (per head) multiplies the scores of a head. A sink
+// (has_sink) is a virtual key of score `sink` without a value: the softmax denominator gains exp(sink). out_scale
+// multiplies the output in both modes.
+//
+// rotary_kv_write: rotation of the channel pairs (2i, 2i + 1), i < ROT / 2, of every q and k head by position *
+// base^(-2i / ROT) (the rest of a head passes unchanged), then q -> q_out and k, v -> their cache slots. The angle is
+// formed and reduced to (-pi, pi] in fp64, sine and cosine are libm sincosf of the reduced angle.
+//
 // headnorm_kv_write: RMS norm of every q head and every k head over its own DK channels (one weight vector of size DK
 // shared by the heads), optionally times a query temperature 1 + coef * ln(floor((p + 1) / every) + 1) of the token's
 // position p, then q -> q_out and k, v -> their cache slots; one wave64 per head.
@@ -233,6 +242,64 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(const TA* __restri
   }
 }
 
+template <typename TI, typename TA>
+__global__ __launch_bounds__(256) void rotary_kv_write_kernel(const TI* __restrict__ q, int ldq, const TI* __restrict__ k,
+                                                              int ldk, const TI* __restrict__ v, int ldv,
+                                                              const int* __restrict__ positions,
+                                                              const int* __restrict__ slots, TA* __restrict__ q_out,
+                                                              TA* __restrict__ k_cache, TA* __restrict__ v_cache, int H,
+                                                              int G, int DK, int DV, int ROT, float base) {
+  extern __shared__ float cs[];  // cos[ROT / 2] | sin[ROT / 2]
+  const int t = blockIdx.x, tid = threadIdx.x, half = ROT >> 1;
+  const double pos = (double)positions[t], l2b = log2((double)base);
+  for (int i = tid; i < half; i += 256) {
+    const double a = pos * exp2(-(double)(2 * i) / (double)ROT * l2b);
+    const double r = a - 6.283185307179586476925 * rint(a * 0.15915494309189533577);
+    float sn, c;
+    sincosf((float)r, &sn, &c);
+    cs[i] = c;
+    cs[half + i] = sn;
+  }
+  __syncthreads();
+  const int slot = slots[t];
+  const size_t page = slot >> 4;
+  const int off = slot & 15, hp = DK >> 1;  // pairs of a head; an odd last channel is handled with the rest
+  const TI* qr = q + (size_t)t * ldq;
+  const TI* kr = k + (size_t)t * ldk;
+  TA* qo = q_out + (size_t)t * H * DK;
+  for (int x = tid; x < (H + G) * hp; x += 256) {
+    const int hh = x / hp, i = x - hh * hp;
+    const bool isq = hh < H;
+    const int g = isq ? hh : hh - H;
+    const TI* src = (isq ? qr : kr) + (size_t)g * DK + 2 * i;
+    TA* dst = isq ? qo + (size_t)g * DK + 2 * i : k_cache + ((page * G + g) * 16 + off) * DK + 2 * i;
+    const float u = (float)src[0], w = (float)src[1];
+    if (i < half) {
+      const float c = cs[i], sn = cs[half + i];
+      dst[0] = (TA)(u * c - w * sn);
+      dst[1] = (TA)(w * c + u * sn);
+    } else {
+      dst[0] = (TA)u;
+      dst[1] = (TA)w;
+    }
+  }
+  if (DK & 1) {
+    for (int hh = tid; hh < H + G; hh += 256) {
+      const bool isq = hh < H;
+      const int g = isq ? hh : hh - H;
+      const TI xv = ((isq ? qr : kr) + (size_t)g * DK)[DK - 1];
+      if (isq) qo[(size_t)g * DK + DK - 1] = (TA)(float)xv;
+      else k_cache[((page * G + g) * 16 + off) * DK + DK - 1] = (TA)(float)xv;
+    }
+  }
+  const int NV = G * DV;
+  const TI* vr = v + (size_t)t * ldv;
+  for (int i = tid; i < NV; i += 256) {
+    const int g = i / DV, c = i - g * DV;
+    v_cache[((page * G + g) * DV + c) * 16 + off] = (TA)(float)vr[i];
+  }
+}
+
 constexpr int kMaxVChunks = 8;  // DV <= 512
 
 template <typename TA, bool SIG>
@@ -241,7 +308,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     const int* __restrict__ block_tables, int maxb, const int* __restrict__ cu_q, const int* __restrict__ ctx, int S,
     TA* __restrict__ out, int ldo, int TH, int H, int G, int DK, int DV, float scale, float softcap, int window,
     const float* __restrict__ r1, const float* __restrict__ r2, const TA* __restrict__ gate, int ldg, int skip_len,
-    const float* __restrict__ sig_bias, float out_scale, int nsplit, float* __restrict__ part) {
+    const float* __restrict__ sig_bias, float out_scale, int nsplit, float* __restrict__ part, int chunk,
+    const float* __restrict__ hscale, int has_sink, float sink) {
   extern __shared__ float lds[];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int th = blockIdx.x * 4 + wid;
@@ -257,7 +325,9 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
   const int s = lo, c0 = cu_q[s];
   if (cu_q[s + 1] - c0 >= skip_len) return;  // long portions run on the matrix-core kernel
   const int pos = ctx[s] - (cu_q[s + 1] - c0) + (t - c0);
-  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  int first = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) first = max(first, pos / chunk * chunk);
+  if (hscale) scale *= hscale[h];
   const TA* qr = q + (size_t)th * DK;
   for (int i = lane; i < DK; i += 64) qs[i] = (float)qr[i];
   __builtin_amdgcn_wave_barrier();
@@ -327,7 +397,15 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     }
     return;
   }
-  const float inv_l = SIG ? out_scale : 1.0f / l;
+  float inv_l = out_scale;
+  if (!SIG) {
+    if (has_sink) {  // a virtual key of score `sink` without a value
+      const float m_fin = fmaxf(m, sink), f = expf(m - m_fin);
+      l = l * f + expf(sink - m_fin);
+      inv_l *= f;
+    }
+    inv_l /= l;
+  }
   TA* o = out + (size_t)t * ldo + (size_t)h * DV;
 #pragma unroll
   for (int n = 0; n < kMaxVChunks; ++n) {
@@ -356,21 +434,22 @@ __global__ __launch_bounds__(256) void sigmoid_split_reduce_kernel(const float* 
 template <typename TA>
 __global__ __launch_bounds__(256) void softmax_split_reduce_kernel(const float* __restrict__ part, int nsplit,
                                                                    TA* __restrict__ out, int ldo, int T, int H, int DV,
-                                                                   const TA* __restrict__ gate, int ldg) {
+                                                                   const TA* __restrict__ gate, int ldg, float out_scale,
+                                                                   int has_sink, float sink) {
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= (long)T * H * DV) return;
   const int th = (int)(e / DV), c = (int)(e % DV), t = th / H, h = th - t * H;
   const size_t TH = (size_t)T * H, W = DV + 2;
-  float M = -INFINITY;
+  float M = has_sink ? sink : -INFINITY;
   for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, part[((size_t)sp * TH + th) * W + DV]);
-  float num = 0.f, den = 0.f;
+  float num = 0.f, den = has_sink ? expf(sink - M) : 0.f;
   for (int sp = 0; sp < nsplit; ++sp) {
     const float* p = part + ((size_t)sp * TH + th) * W;
     const float f = expf(p[DV] - M);
     num = fmaf(p[c], f, num);
     den = fmaf(p[DV + 1], f, den);
   }
-  float y = num / den;
+  float y = num / den * out_scale;
   if (gate) y *= 1.0f / (1.0f + expf(-(float)gate[(size_t)t * ldg + (size_t)h * DV + c]));
   out[(size_t)t * ldo + (size_t)h * DV + c] = (TA)y;
 }
@@ -412,10 +491,11 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
     const int* __restrict__ block_tables, int maxb, const int* __restrict__ cu_q, const int* __restrict__ ctx, int S,
     bf16* __restrict__ out, int ldo, int H, int G, float scale, float softcap, int window, const float* __restrict__ r1,
     const float* __restrict__ r2, const bf16* __restrict__ gate, int ldg, const float* __restrict__ sig_bias,
-    float out_scale) {
+    float out_scale, int chunk, const float* __restrict__ hscale, int has_sink, float sink) {
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int h = blockIdx.y * 4 + wid;
   if (h >= H) return;
+  if (hscale) scale *= hscale[h];
   // tile -> (sequence, first row): sequences of at least kMfmaMinLen rows own ceil(len / 32) tiles each
   int s = 0, seen = 0, len = 0;
   for (; s < S; ++s) {
@@ -431,7 +511,9 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
   const int t = cu_q[s] + row0 + min(qi, nrows - 1);
   const int pos0 = ctx[s] - len + row0;             // position of the tile's first query
   const int pos = pos0 + min(qi, nrows - 1), last = pos0 + nrows - 1;
-  const int first = window > 0 ? max(0, pos0 - window + 1) : 0;
+  int first = window > 0 ? max(0, pos0 - window + 1) : 0;
+  if (chunk > 0) first = max(first, pos0 / chunk * chunk);
+  const int qfirst = chunk > 0 ? pos / chunk * chunk : 0;  // the first key this lane's query sees in chunk mode
   const int* bt = block_tables + (size_t)s * maxb;
   bf16x8 qf[DK / 16];
   const bf16* qr = q + ((size_t)t * H + h) * DK + 8 * hb;
@@ -458,7 +540,7 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
       float x = sc[r] * scale;
       if (softcap > 0.f) x = softcap * tanh_fast(x * inv_cap);
       if (r1) x -= b1 * (0.6931471805599453f * __builtin_amdgcn_logf(fmaf(b2, (float)max(dist, 0), 1.0f)));
-      const bool ok = valid && dist >= 0 && (window <= 0 || dist < window);
+      const bool ok = valid && dist >= 0 && (window <= 0 || dist < window) && pos - dist >= qfirst;
       x = ok ? x : kMasked;
       sc[r] = x;
       mt = fmaxf(mt, x);
@@ -507,9 +589,17 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
       }
     }
   }
-  const float l = sum_halves(l_run);
+  float l = sum_halves(l_run);
   if (!valid) return;
-  const float inv_l = SIG ? out_scale : 1.0f / l;
+  float inv_l = out_scale;
+  if (!SIG) {
+    if (has_sink) {  // a virtual key of score `sink` without a value
+      const float m_fin = fmaxf(m_run, sink), f = expf(m_run - m_fin);
+      l = l * f + expf(sink - m_fin);
+      inv_l *= f;
+    }
+    inv_l /= l;
+  }
   bf16* o = out + (size_t)t * ldo + (size_t)h * DV;
   const bf16* gr = gate ? gate + (size_t)t * ldg + (size_t)h * DV : nullptr;
 #pragma unroll
@@ -533,16 +623,17 @@ template <int DK, int DV>
 void launch_window_mfma(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int maxb,
                         const int* cu_q, const int* ctx, int S, void* out, int ldo, int T, int H, int G, float scale,
                         float softcap, int window, const float* r1, const float* r2, const void* gate, int ldg,
-                        const float* sig_bias, int sig, float out_scale, hipStream_t st) {
+                        const float* sig_bias, int sig, float out_scale, hipStream_t st, int chunk, const float* hscale,
+                        int has_sink, float sink) {
   const dim3 grid((T + kTileQ - 1) / kTileQ + S, (H + 3) / 4);
   if (sig)
     window_attention_mfma_kernel<DK, DV, true><<<grid, 256, 0, st>>>(
         (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, maxb, cu_q, ctx, S, (bf16*)out, ldo, H,
-        G, scale, softcap, window, r1, r2, (const bf16*)gate, ldg, sig_bias, out_scale);
+        G, scale, softcap, window, r1, r2, (const bf16*)gate, ldg, sig_bias, out_scale, chunk, hscale, has_sink, sink);
   else
     window_attention_mfma_kernel<DK, DV, false><<<grid, 256, 0, st>>>(
         (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, maxb, cu_q, ctx, S, (bf16*)out, ldo, H,
-        G, scale, softcap, window, r1, r2, (const bf16*)gate, ldg, sig_bias, out_scale);
+        G, scale, softcap, window, r1, r2, (const bf16*)gate, ldg, sig_bias, out_scale, chunk, hscale, has_sink, sink);
 }
 
 }  // namespace
@@ -597,6 +688,23 @@ void gai_latent_kv_write(const void* q, int ldq, const void* dkv, int ldk, const
   GAI_LAUNCH_CHECK();
 }
 
+// dt_in / dt: 0 = bf16, 1 = fp32 (inputs may be fp32 while the cache is bf16: the output of an fp32 convolution)
+void gai_rotary_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const int* positions,
+                         const int* slots, void* q_out, void* k_cache, void* v_cache, int T, int H, int G, int DK, int DV,
+                         int ROT, float base, int dt_in, int dt, hipStream_t st) {
+  if (T == 0) return;
+  if (ROT % 2 || ROT < 0 || ROT > DK) gai_launch_error(__FILE__, __LINE__, "rotary_kv_write: an even number of rotated channels within a head");
+  if (!dt_in && dt) gai_launch_error(__FILE__, __LINE__, "rotary_kv_write: bf16 inputs go with a bf16 cache");
+  const size_t lds = (size_t)(ROT > 0 ? ROT : 1) * sizeof(float);
+#define GAI_ROT(TI, TA)                                                                                              \
+  rotary_kv_write_kernel<TI, TA><<<T, 256, lds, st>>>((const TI*)q, ldq, (const TI*)k, ldk, (const TI*)v, ldv, positions, \
+                                                      slots, (TA*)q_out, (TA*)k_cache, (TA*)v_cache, H, G, DK, DV, ROT, \
+                                                      base)
+  if (dt_in && dt) GAI_ROT(float, float); else if (dt_in) GAI_ROT(float, bf16); else GAI_ROT(bf16, bf16);
+#undef GAI_ROT
+  GAI_LAUNCH_CHECK();
+}
+
 // Key splits of a decode step (every row a single token): enough waves to give each SIMD a few
 int gai_sigmoid_attention_splits(int T, int S, int H) {
   if (T != S || T * H >= 2048) return 1;
@@ -608,8 +716,10 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
                           const int* cu_q, const int* ctx, int S, void* out, int ldo, int T, int H, int G, int DK, int DV,
                           float scale, float softcap, int window, const float* r1, const float* r2, const void* gate,
                           int ldg, const float* sig_bias, int sig, float out_scale, int dt, hipStream_t st,
-                          float* part) {
+                          float* part, int chunk, const float* hscale, int has_sink, float sink) {
   if (T == 0 || S == 0) return;
+  if (sig && (chunk > 0 || hscale || has_sink))
+    gai_launch_error(__FILE__, __LINE__, "window_attention: chunks, head scales and sinks go with the softmax mode");
   if (DV > 64 * kMaxVChunks) gai_launch_error(__FILE__, __LINE__, "window_attention: value head size above 512");
   if (H % G) gai_launch_error(__FILE__, __LINE__, "window_attention: heads must be a multiple of kv heads");
   const int TH = T * H, grid = (TH + 3) / 4;
@@ -621,7 +731,8 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
 #define GAI_WIN(K_, V_)                                                                                              \
   if (DK == K_ && DV == V_) {                                                                                        \
     launch_window_mfma<K_, V_>(q, k_cache, v_cache, block_tables, maxb, cu_q, ctx, S, out, ldo, T, H, G, scale,      \
-                               softcap, window, r1, r2, gate, ldg, sig_bias, sig, out_scale, st);                     \
+                               softcap, window, r1, r2, gate, ldg, sig_bias, sig, out_scale, st, chunk, hscale,       \
+                               has_sink, sink);                                                                      \
     skip_len = kMfmaMinLen;                                                                                          \
   }
     GAI_WIN(64, 64) GAI_WIN(64, 128) GAI_WIN(128, 64) GAI_WIN(128, 128) GAI_WIN(256, 256)
@@ -634,7 +745,8 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
 #define GAI_ROW(TA, SIG_)                                                                                            \
   window_attention_kernel<TA, SIG_><<<dim3(grid, nsplit), 256, lds, st>>>(                                           \
       (const TA*)q, (const TA*)k_cache, (const TA*)v_cache, block_tables, maxb, cu_q, ctx, S, (TA*)out, ldo, TH, H, G, \
-      DK, DV, scale, softcap, window, r1, r2, (const TA*)gate, ldg, skip_len, sig_bias, out_scale, nsplit, part)
+      DK, DV, scale, softcap, window, r1, r2, (const TA*)gate, ldg, skip_len, sig_bias, out_scale, nsplit, part,    \
+      chunk, hscale, has_sink, sink)
   if (dt) {
     if (sig) GAI_ROW(float, true); else GAI_ROW(float, false);
   } else {
@@ -645,10 +757,12 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
     const long n = (long)T * H * DV;
     if (dt)
       softmax_split_reduce_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(part, nsplit, (float*)out, ldo, T, H,
-                                                                                       DV, (const float*)gate, ldg);
+                                                                                       DV, (const float*)gate, ldg,
+                                                                                       out_scale, has_sink, sink);
     else
       softmax_split_reduce_kernel<bf16><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(part, nsplit, (bf16*)out, ldo, T, H,
-                                                                                      DV, (const bf16*)gate, ldg);
+                                                                                      DV, (const bf16*)gate, ldg,
+                                                                                      out_scale, has_sink, sink);
   } else if (nsplit > 1) {
     const long n = (long)T * H * DV;
     if (dt)

@@ -17,6 +17,10 @@
 // moe_route (choice bias): the experts are chosen by softmax score + bias_e while the weights stay the plain scores,
 //              renormalised over the chosen ones (+ eps in the sum); libm expf, all fp32.
 // moe_combine (identity experts): a chosen id >= n_real has no weights - its output is the token's own input row.
+// moe_route (grouped sigmoid): choice on sigmoid score + bias among the experts of the best groups (a group scores the
+//              sum of its two largest choice scores); weights = the chosen plain scores renormalised (+ eps), scaled.
+// moe_gemm (clamped gated): g = min(gate, p), u = clamp(up, +-p), g sigmoid(1.702 g) (u + 1) on [gate16 | up16] rows.
+// moe_combine (residual gate): the residual row (a shared expert's output) times sigmoid of a per-token logit.
 // moe_scale_rows: expert-sorted copies of the token rows, each times its routing weight (experts whose routing weight
 //              multiplies the INPUT of a non-linear expert).
 #include "gai_common.h"
@@ -74,14 +78,87 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int T, int E,
   }
 }
 
+constexpr float kGluSlope = 1.702f;  // slope of the sigmoid in the clamped gated activation
+
+// gate / up pair -> activation: SwiGLU (ACT 1) or the clamped gated form (ACT 3, limit p)
+template <int ACT>
+__device__ __forceinline__ float glu_pair(float g, float u, float p) {
+  if (ACT == 3) {
+    g = fminf(g, p);
+    u = fminf(fmaxf(u, -p), p);
+    return g / (1.0f + expf(-kGluSlope * g)) * (u + 1.0f);
+  }
+  return silu(g) * u;
+}
+
+// Sigmoid scores with a choice correction and group-limited top-k, one lane per token: choice score c_e = sigmoid(x_e) +
+// bias_e; the experts form NG equal groups of neighbours, a group scores the sum of its two largest choice scores, only
+// experts of the KEEP best groups can be chosen (NG <= 64: the kept groups are a bit mask); the weights are the chosen
+// plain scores over their sum (+ eps), times scale. All fp32, libm expf.
+__global__ void moe_route_grouped_kernel(const float* __restrict__ logits, int T, int E, int k, int* __restrict__ ids,
+                                         float* __restrict__ w, const float* __restrict__ bias, float eps, int NG,
+                                         int KEEP, float scale) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* x = logits + (size_t)t * E;
+  const int per = E / NG;
+  unsigned long long kept = ~0ull;
+  if (NG > 1 && KEEP < NG) {
+    float gs[64];
+    for (int g = 0; g < NG; ++g) {
+      float a = -INFINITY, b = -INFINITY;  // the two largest of the group
+      for (int e = g * per; e < (g + 1) * per; ++e) {
+        const float c = 1.0f / (1.0f + expf(-x[e])) + (bias ? bias[e] : 0.f);
+        if (c > a) { b = a; a = c; } else if (c > b) b = c;
+      }
+      gs[g] = per > 1 ? a + b : a;
+    }
+    kept = 0ull;
+    for (int n = 0; n < KEEP; ++n) {
+      int best = -1;
+      float bvv = -INFINITY;
+      for (int g = 0; g < NG; ++g)
+        if (!((kept >> g) & 1ull) && (best < 0 || gs[g] > bvv)) { best = g; bvv = gs[g]; }
+      kept |= 1ull << best;
+    }
+  }
+  float bv[16];
+  int bi[16];
+  for (int j = 0; j < k; ++j) { bv[j] = -INFINITY; bi[j] = -1; }
+  for (int e = 0; e < E; ++e) {
+    if (!((kept >> (e / per)) & 1ull)) continue;
+    const float p = 1.0f / (1.0f + expf(-x[e])) + (bias ? bias[e] : 0.f);
+    if (p > bv[k - 1] || bi[k - 1] < 0) {
+      int j = k - 1;
+      while (j > 0 && (bi[j - 1] < 0 || bv[j - 1] < p)) {
+        bv[j] = bv[j - 1];
+        bi[j] = bi[j - 1];
+        --j;
+      }
+      bv[j] = p;
+      bi[j] = e;
+    }
+  }
+  float tot = eps;
+  for (int j = 0; j < k; ++j) {
+    bi[j] = bi[j] < 0 ? 0 : bi[j];
+    bv[j] = 1.0f / (1.0f + expf(-x[bi[j]]));  // the weights are the plain scores
+    tot += bv[j];
+  }
+  for (int j = 0; j < k; ++j) {
+    ids[(size_t)t * k + j] = bi[j];
+    w[(size_t)t * k + j] = bv[j] / tot * scale;
+  }
+}
+
 __device__ __forceinline__ void glds16(const void* g, char* lds) {
   __builtin_amdgcn_global_load_lds(g, GAI_LDS(lds), 16, 0, 0);
 }
 
-template <int ACT>  // 0 none, 1 SwiGLU, 2 squared ReLU
+template <int ACT>  // 0 none, 1 SwiGLU, 2 squared ReLU, 3 clamped gated (limit actp)
 __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const bf16* __restrict__ A, const int* __restrict__ a_rows,
                                                           const bf16* __restrict__ W, bf16* __restrict__ C,
-                                                          const int* __restrict__ offs, int E, int N, int K) {
+                                                          const int* __restrict__ offs, int E, int N, int K, float actp) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   // ---- which (expert, row tile) is this block?
   int t = blockIdx.x, e = 0, r0 = 0, rend = 0;
@@ -167,7 +244,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const bf16* __restrict
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
-  constexpr bool SWIGLU = ACT == 1;
+  constexpr bool SWIGLU = ACT == 1 || ACT == 3;  // gate / up pairs in [gate16 | up16] row blocks
   const int ldc = SWIGLU ? N / 2 : N;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -179,7 +256,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const bf16* __restrict
 #pragma unroll
         for (int jp = 0; jp < 2; ++jp) {
           const int nout = (n0 + wn * 64) / 2 + 16 * jp + (lane & 15);
-          if (2 * nout < N) C[(size_t)m * ldc + nout] = (bf16)(silu(acc[i][2 * jp][r]) * acc[i][2 * jp + 1][r]);
+          if (2 * nout < N) C[(size_t)m * ldc + nout] = (bf16)glu_pair<ACT>(acc[i][2 * jp][r], acc[i][2 * jp + 1][r], actp);
         }
       } else {
 #pragma unroll
@@ -199,7 +276,8 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const bf16* __restrict
 template <typename TA, int ACT>
 __global__ __launch_bounds__(256) void moe_gemm_generic_kernel(const TA* __restrict__ A, const int* __restrict__ a_rows,
                                                                const TA* __restrict__ W, TA* __restrict__ C,
-                                                               const int* __restrict__ offs, int E, int N, int K) {
+                                                               const int* __restrict__ offs, int E, int N, int K,
+                                                               float actp) {
   constexpr int TM = 32, TN = 64, TK = 32;
   __shared__ float As[TM][TK + 1];
   __shared__ float Ws[TN][TK + 1];
@@ -255,10 +333,11 @@ __global__ __launch_bounds__(256) void moe_gemm_generic_kernel(const TA* __restr
     for (int c = 0; c < 4; ++c) {
       const int n = n0 + tx + 16 * c;
       float v = acc[r][c];
-      if (ACT == 1) {  // rows interleaved [gate16 | up16]: columns c = 0, 2 are gates, c + 1 their up partners
+      if (ACT == 1 || ACT == 3) {  // rows interleaved [gate16 | up16]: columns c = 0, 2 are gates, c + 1 their up partners
         if ((c & 1) == 0 && n + 16 < N) {
-          const float g = v;
-          C[(size_t)m * (N / 2) + n0 / 2 + tx + 16 * (c >> 1)] = (TA)(g / (1.0f + expf(-g)) * acc[r][c + 1]);
+          const float g = v, u = acc[r][c + 1];
+          C[(size_t)m * (N / 2) + n0 / 2 + tx + 16 * (c >> 1)] =
+              (TA)(ACT == 1 ? g / (1.0f + expf(-g)) * u : glu_pair<3>(g, u, actp));
         }
         continue;
       }
@@ -273,7 +352,8 @@ __global__ __launch_bounds__(256) void moe_combine_generic_kernel(const TA* __re
                                                                   const float* __restrict__ w, const TA* residual,
                                                                   TA* __restrict__ out, int T, int k, int D,
                                                                   const int* __restrict__ ids, int n_real,
-                                                                  const TA* __restrict__ ident) {
+                                                                  const TA* __restrict__ ident,
+                                                                  const TA* __restrict__ rgate, int ldrg) {
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= (long)T * D) return;
   const int t = (int)(e / D), d = (int)(e % D);
@@ -283,7 +363,10 @@ __global__ __launch_bounds__(256) void moe_combine_generic_kernel(const TA* __re
     const float y = idn ? (float)ident[(size_t)t * D + d] : (float)Y[(size_t)pos[(size_t)t * k + j] * D + d];
     acc += w ? w[(size_t)t * k + j] * y : y;
   }
-  if (residual) acc += (float)residual[(size_t)t * D + d];
+  if (residual) {
+    const float rg = rgate ? 1.0f / (1.0f + expf(-(float)rgate[(size_t)t * ldrg])) : 1.0f;
+    acc += rg * (float)residual[(size_t)t * D + d];
+  }
   out[(size_t)t * D + d] = (TA)acc;
 }
 
@@ -302,7 +385,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const bf16* __restrict
                                                           const float* __restrict__ w, const bf16* residual,
                                                           bf16* __restrict__ out, int T, int k, int D,
                                                           const int* __restrict__ ids, int n_real,
-                                                          const bf16* __restrict__ ident) {
+                                                          const bf16* __restrict__ ident,
+                                                          const bf16* __restrict__ rgate, int ldrg) {
   const int units = D / 8;
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= (long)T * units) return;
@@ -317,8 +401,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const bf16* __restrict
   }
   if (residual) {
     const bf16x8 r = load8(residual + (size_t)t * D + u * 8);
+    const float rg = rgate ? 1.0f / (1.0f + expf(-(float)rgate[(size_t)t * ldrg])) : 1.0f;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) acc[q] += (float)r[q];
+    for (int q = 0; q < 8; ++q) acc[q] += rg * (float)r[q];
   }
   bf16x8 o;
 #pragma unroll
@@ -494,26 +579,42 @@ void gai_moe_scale_rows(const void* h, const int* pos, const float* w, void* out
   GAI_LAUNCH_CHECK();
 }
 
+void gai_moe_route_grouped(const float* logits, int T, int E, int k, int* ids, float* w, const float* bias, float eps,
+                           int NG, int KEEP, float scale, hipStream_t st) {
+  if (T == 0) return;
+  if (NG < 1 || NG > 64 || E % NG || KEEP < 1 || KEEP > NG)
+    gai_launch_error(__FILE__, __LINE__, "moe_route: 1 <= keep <= groups <= 64 equal groups of experts");
+  if (k < 1 || k > 16 || k > E / NG * KEEP)
+    gai_launch_error(__FILE__, __LINE__, "moe_route: 1 <= top-k <= min(16, experts of the kept groups)");
+  moe_route_grouped_kernel<<<(T + 255) / 256, 256, 0, st>>>(logits, T, E, k, ids, w, bias, eps, NG, KEEP, scale);
+  GAI_LAUNCH_CHECK();
+}
+
 void gai_moe_gemm(const void* A, const int* a_rows, const void* W, void* C, const int* offs, int E, int rows_total,
-                  int N, int K, int act, hipStream_t st, int dt) {
+                  int N, int K, int act, hipStream_t st, int dt, float actp) {
   if (rows_total == 0) return;
-  if (act < 0 || act > 2) gai_launch_error(__FILE__, __LINE__, "moe_gemm: act 0 (none), 1 (SwiGLU) or 2 (squared ReLU)");
+  if (act < 0 || act > 3)
+    gai_launch_error(__FILE__, __LINE__, "moe_gemm: act 0 (none), 1 (SwiGLU), 2 (squared ReLU) or 3 (clamped gated)");
   if (dt || K % MBK) {  // fp32 operands, or K off the MFMA tile grid: the generic grouped kernel
-    if (act == 1 && N % 32) gai_launch_error(__FILE__, __LINE__, "moe_gemm: SwiGLU rows come in [gate16 | up16] blocks");
+    if ((act == 1 || act == 3) && N % 32)
+      gai_launch_error(__FILE__, __LINE__, "moe_gemm: gated rows come in [gate16 | up16] blocks");
     const dim3 grid((rows_total + 31) / 32 + E, (N + 63) / 64);
 #define GAI_MG(TA, ACT_)                                                                                        \
-  moe_gemm_generic_kernel<TA, ACT_><<<grid, 256, 0, st>>>((const TA*)A, a_rows, (const TA*)W, (TA*)C, offs, E, N, K)
+  moe_gemm_generic_kernel<TA, ACT_><<<grid, 256, 0, st>>>((const TA*)A, a_rows, (const TA*)W, (TA*)C, offs, E, N, K, actp)
     if (dt) {
-      if (act == 2) GAI_MG(float, 2); else if (act == 1) GAI_MG(float, 1); else GAI_MG(float, 0);
+      if (act == 3) GAI_MG(float, 3); else if (act == 2) GAI_MG(float, 2); else if (act == 1) GAI_MG(float, 1);
+      else GAI_MG(float, 0);
     } else {
-      if (act == 2) GAI_MG(bf16, 2); else if (act == 1) GAI_MG(bf16, 1); else GAI_MG(bf16, 0);
+      if (act == 3) GAI_MG(bf16, 3); else if (act == 2) GAI_MG(bf16, 2); else if (act == 1) GAI_MG(bf16, 1);
+      else GAI_MG(bf16, 0);
     }
 #undef GAI_MG
     GAI_LAUNCH_CHECK();
     return;
   }
   // decode steps (<= 64 expert rows in all): every expert's weights streamed once by the decode kernel
-  if (gai_moe_gemm_dec2(A, a_rows, W, C, offs, E, rows_total, N, K, act, st)) return;
+  // (the clamped gated epilogue lives in the tiled kernels only)
+  if (act != 3 && gai_moe_gemm_dec2(A, a_rows, W, C, offs, E, rows_total, N, K, act, st)) return;
   const dim3 grid((rows_total + MBM - 1) / MBM + E, (N + MBN - 1) / MBN);
   const int lds = 4 * kMTile;
   static bool once = false;
@@ -521,34 +622,41 @@ void gai_moe_gemm(const void* A, const int* a_rows, const void* W, void* C, cons
     hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_kernel<0>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_kernel<3>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     once = true;
   }
   if (act == 1) {
-    moe_gemm_kernel<1><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K);
+    moe_gemm_kernel<1><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K, actp);
   } else if (act == 2) {
-    moe_gemm_kernel<2><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K);
+    moe_gemm_kernel<2><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K, actp);
+  } else if (act == 3) {
+    moe_gemm_kernel<3><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K, actp);
   } else {
-    moe_gemm_kernel<0><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K);
+    moe_gemm_kernel<0><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K, actp);
   }
   GAI_LAUNCH_CHECK();
 }
 
 void gai_moe_combine(const void* Y, const int* pos, const float* w, const void* residual, void* out, int T, int k,
-                     int D, hipStream_t st, int dt, const int* ids, int n_real, const void* ident) {
+                     int D, hipStream_t st, int dt, const int* ids, int n_real, const void* ident, const void* rgate,
+                     int ldrg) {
   if (T == 0) return;
   if (dt || D % 8 || !w) {
     const long n = (long)T * D;
     if (dt)
       moe_combine_generic_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(
-          (const float*)Y, pos, w, (const float*)residual, (float*)out, T, k, D, ids, n_real, (const float*)ident);
+          (const float*)Y, pos, w, (const float*)residual, (float*)out, T, k, D, ids, n_real, (const float*)ident,
+          (const float*)rgate, ldrg);
     else
       moe_combine_generic_kernel<bf16><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(
-          (const bf16*)Y, pos, w, (const bf16*)residual, (bf16*)out, T, k, D, ids, n_real, (const bf16*)ident);
+          (const bf16*)Y, pos, w, (const bf16*)residual, (bf16*)out, T, k, D, ids, n_real, (const bf16*)ident,
+          (const bf16*)rgate, ldrg);
     GAI_LAUNCH_CHECK();
     return;
   }
   const long n = (long)T * (D / 8);
   moe_combine_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const bf16*)Y, pos, w, (const bf16*)residual,
-                                                                   (bf16*)out, T, k, D, ids, n_real, (const bf16*)ident);
+                                                                   (bf16*)out, T, k, D, ids, n_real, (const bf16*)ident,
+                                                                   (const bf16*)rgate, ldrg);
   GAI_LAUNCH_CHECK();
 }

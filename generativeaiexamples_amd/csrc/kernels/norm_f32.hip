@@ -5,13 +5,14 @@
 //   poly_norm         y = a N(z) + b N(z^2) + c N(z^3) + e,  N(t) = t * rsqrt(mean(t^2) + eps) over the row
 //   head_norm_gate    y = o * rsqrt(mean_head(o^2) + eps) * nw * act(gate)   (act: silu | sigmoid), one head per wave
 //   embed_scale_f32   out = table[id] * scale as fp32 (+ pos_table[position]: learned absolute positions)
-//   gated_norm_add    g = y * sigmoid(gate);  res += g * rsqrt(mean(g^2) + eps) * wpost;  out = rmsnorm(res) * wnext
+//   gated_norm_add    g = y * sigmoid(gate) (gate = nullptr: g = y);  res += g * rsqrt(mean(g^2) + eps) * wpost;  out = rmsnorm(res) * wnext
 //                     (post-norm gated residual: the closing norm of a sublayer, the residual add and the opening norm
 //                     of the next sublayer in one pass)
 //   gate_group_norm   g = y * silu(z);  out = g * rsqrt(mean_group(g^2) + eps) * w, the row cut into equal groups
 //   add_dyt_f32       res += delta (+ extra);  out = tanh(alpha * res) * w + b   (dynamic tanh: a norm without statistics,
 //                     so the pass is purely element-wise: four elements per thread, no reduction)
-//   act_mul           out = act(a) (* b), act: silu | squared ReLU | cap * tanh(a / cap); fp32 arithmetic, a / b column
+//   act_mul           out = act(a) (* b), act: silu | squared ReLU | cap * tanh(a / cap) | tanh GELU, or the clamped gated
+//                     activation min(a, cap) * sigmoid(1.702 min(a, cap)) * (clamp(b, +-cap) + 1); fp32 arithmetic, a / b column
 //                     slices of wider rows, out bf16 or fp32
 //
 // Activations (delta, z, gate, out, y) are bf16 or fp32 (template TA); every statistic and product is fp32.
@@ -84,7 +85,8 @@ __global__ __launch_bounds__(256) void poly_norm_kernel(const TA* __restrict__ z
 template <typename TA>
 __global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(const float* __restrict__ o, const TA* __restrict__ gate,
                                                                   int ldg, const float* __restrict__ nw, int nw_per_head,
-                                                                  int act, TA* __restrict__ y, int H, int DV, float eps) {
+                                                                  int act, TA* __restrict__ y, int ldy, int H, int DV,
+                                                                  float eps) {
   constexpr int kMax = 32;  // DV <= 8192
   __shared__ float scratch[16];
   const int th = blockIdx.x, t = th / H, h = th % H, tid = threadIdx.x;
@@ -101,7 +103,7 @@ __global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(const float* _
   const float inv = 1.0f / sqrtf(s / DV + eps);
   const TA* g = gate + (size_t)t * ldg + (size_t)h * DV;
   const float* wr = nw + (nw_per_head ? (size_t)h * DV : 0);
-  TA* yr = y + (size_t)th * DV;
+  TA* yr = y + (size_t)t * ldy + (size_t)h * DV;
 #pragma unroll
   for (int q = 0; q < kMax; ++q) {
     const int i = tid + 256 * q;
@@ -116,8 +118,8 @@ __global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(const float* _
 template <typename TA>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const TA* __restrict__ gate,
                                                              int ldg, const float* __restrict__ nw, int nw_per_head,
-                                                             int act, TA* __restrict__ y, int TH, int H, int DV,
-                                                             float eps) {
+                                                             int act, TA* __restrict__ y, int ldy, int TH, int H,
+                                                             int DV, float eps) {
   const int lane = threadIdx.x & 63;
   const int th = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (th >= TH) return;
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   const float inv = 1.0f / sqrtf(s / DV + eps);
   const TA* g = gate + (size_t)t * ldg + (size_t)h * DV;
   const float* wr = nw + (nw_per_head ? (size_t)h * DV : 0);
-  TA* yr = y + (size_t)th * DV;
+  TA* yr = y + (size_t)t * ldy + (size_t)h * DV;
   for (int i = lane; i < DV; i += 64) {
     const float gv = (float)g[i];
     const float sg = 1.0f / (1.0f + expf(-gv));
@@ -173,14 +175,14 @@ __global__ __launch_bounds__(256) void gated_norm_add_kernel(float* __restrict__
   const TG* gr = gate + (size_t)row * ldg;
   float s = 0.f;
   for (int i = lane; i < D; i += 64) {
-    const float g = (float)yr[i] / (1.0f + expf(-(float)gr[i]));
+    const float g = gate ? (float)yr[i] / (1.0f + expf(-(float)gr[i])) : (float)yr[i];
     s += g * g;
   }
   s = wave_sum(s);
   const float inv = 1.0f / sqrtf(s / D + eps);
   float s2 = 0.f;
   for (int i = lane; i < D; i += 64) {
-    const float g = (float)yr[i] / (1.0f + expf(-(float)gr[i]));
+    const float g = gate ? (float)yr[i] / (1.0f + expf(-(float)gr[i])) : (float)yr[i];
     const float v = r[i] + g * inv * wpost[i];
     r[i] = v;
     s2 += v * v;
@@ -216,11 +218,11 @@ __global__ __launch_bounds__(256) void gated_norm_add_wide_kernel(float* __restr
 #pragma unroll
   for (int q = 0; q < kWideRegs; ++q) {
     const int i = tid + 256 * q;
-    g[q] = i < D ? (float)yr[i] / (1.0f + expf(-(float)gr[i])) : 0.f;
+    g[q] = i < D ? (gate ? (float)yr[i] / (1.0f + expf(-(float)gr[i])) : (float)yr[i]) : 0.f;
     s += g[q] * g[q];
   }
   for (int i = tid + 256 * kWideRegs; i < D; i += 256) {
-    const float v = (float)yr[i] / (1.0f + expf(-(float)gr[i]));
+    const float v = gate ? (float)yr[i] / (1.0f + expf(-(float)gr[i])) : (float)yr[i];
     s += v * v;
   }
   s = block_sum(s, scratch);
@@ -236,7 +238,7 @@ __global__ __launch_bounds__(256) void gated_norm_add_wide_kernel(float* __restr
     }
   }
   for (int i = tid + 256 * kWideRegs; i < D; i += 256) {
-    const float v = r[i] + (float)yr[i] / (1.0f + expf(-(float)gr[i])) * inv * wpost[i];
+    const float v = r[i] + (gate ? (float)yr[i] / (1.0f + expf(-(float)gr[i])) : (float)yr[i]) * inv * wpost[i];
     r[i] = v;
     s2 += v * v;
   }
@@ -358,6 +360,8 @@ __global__ __launch_bounds__(256) void add_dyt_f32_kernel(float* __restrict__ re
   for (int i = 0; i < VEC; ++i) o[i] = (TA)fmaf(tanhf(alpha * v[i]), w[c0 + i], b[c0 + i]);
 }
 
+constexpr float kGluSlope = 1.702f;  // slope of the sigmoid in the clamped gated activation
+
 template <typename TI, typename TO, int VEC>
 __global__ __launch_bounds__(256) void act_mul_kernel(const TI* __restrict__ a, int lda, const TI* __restrict__ b, int ldb,
                                                       TO* __restrict__ out, int T, int C, int act, float cap) {
@@ -377,8 +381,13 @@ __global__ __launch_bounds__(256) void act_mul_kernel(const TI* __restrict__ a, 
     float y;
     if (act == 0) y = x / (1.0f + expf(-x));
     else if (act == 1) y = fmaxf(x, 0.f) * fmaxf(x, 0.f);
-    else y = cap * tanhf(x / cap);
-    if (b) y *= (float)xb.v[i];
+    else if (act == 2) y = cap * tanhf(x / cap);
+    else if (act == 3) y = 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+    else {  // clamped gated activation of (a, b) with limit cap
+      const float g = fminf(x, cap), u = fminf(fmaxf((float)xb.v[i], -cap), cap);
+      y = g / (1.0f + expf(-kGluSlope * g)) * (u + 1.0f);
+    }
+    if (b && act != 4) y *= (float)xb.v[i];
     yo.v[i] = (TO)y;
   }
   *reinterpret_cast<VO*>(out + (size_t)row * C + c) = yo;
@@ -410,25 +419,25 @@ void gai_poly_norm(const void* z, void* y, const float* coef, int T, int F, floa
 }
 
 void gai_head_norm_gate(const float* o, const void* gate, int ldg, const float* nw, int nw_per_head, int act, void* y,
-                        int T, int H, int DV, float eps, int dt, hipStream_t st) {
+                        int ldy, int T, int H, int DV, float eps, int dt, hipStream_t st) {
   if (T == 0) return;
   const int TH = T * H, grid = (TH + 3) / 4;
   if (TH <= 256 && DV >= 1024 && DV <= 8192) {  // few wide rows: a single wave per row would walk it alone
     if (dt)
       head_norm_gate_wide_kernel<float><<<TH, 256, 0, st>>>(o, (const float*)gate, ldg, nw, nw_per_head, act, (float*)y,
-                                                            H, DV, eps);
+                                                            ldy, H, DV, eps);
     else
-      head_norm_gate_wide_kernel<bf16><<<TH, 256, 0, st>>>(o, (const bf16*)gate, ldg, nw, nw_per_head, act, (bf16*)y, H,
-                                                           DV, eps);
+      head_norm_gate_wide_kernel<bf16><<<TH, 256, 0, st>>>(o, (const bf16*)gate, ldg, nw, nw_per_head, act, (bf16*)y, ldy,
+                                                           H, DV, eps);
     GAI_LAUNCH_CHECK();
     return;
   }
   if (dt)
-    head_norm_gate_kernel<float><<<grid, 256, 0, st>>>(o, (const float*)gate, ldg, nw, nw_per_head, act, (float*)y, TH,
-                                                        H, DV, eps);
+    head_norm_gate_kernel<float><<<grid, 256, 0, st>>>(o, (const float*)gate, ldg, nw, nw_per_head, act, (float*)y, ldy,
+                                                        TH, H, DV, eps);
   else
-    head_norm_gate_kernel<bf16><<<grid, 256, 0, st>>>(o, (const bf16*)gate, ldg, nw, nw_per_head, act, (bf16*)y, TH, H,
-                                                       DV, eps);
+    head_norm_gate_kernel<bf16><<<grid, 256, 0, st>>>(o, (const bf16*)gate, ldg, nw, nw_per_head, act, (bf16*)y, ldy, TH,
+                                                       H, DV, eps);
   GAI_LAUNCH_CHECK();
 }
 
@@ -458,7 +467,9 @@ void gai_gated_norm_add_f32(float* res, const void* y, int ldy, int dt_y, const 
   else                                                                                                               \
     gated_norm_add_kernel<TY, TG, TA><<<grid, 256, 0, st>>>(res, (const TY*)y, ldy, (const TG*)gate, ldg, wpost,     \
                                                             wnext, (TA*)out, T, D, eps)
+  if (!gate) dt_gate = dt_y;  // no gate: the gate type is not read
   if (dt_y && dt_gate && (dt_out || !out)) { GAI_GNA(float, float, float); }
+  else if (dt_y && dt_gate) { GAI_GNA(float, float, bf16); }
   else if (!dt_y && !dt_gate && (!dt_out || !out)) { GAI_GNA(bf16, bf16, bf16); }
   else if (!dt_y && dt_gate && (!dt_out || !out)) { GAI_GNA(bf16, float, bf16); }
   else gai_launch_error(__FILE__, __LINE__, "gated_norm_add_f32: unsupported dtype combination");
@@ -509,8 +520,10 @@ void gai_add_dyt_f32(float* res, const void* delta, int ldd, const float* extra,
 void gai_act_mul(const void* a, int lda, const void* b, int ldb, void* out, int T, int C, int act, float cap, int dt_in,
                  int dt_out, hipStream_t st) {
   if (T == 0 || C == 0) return;
-  if (act < 0 || act > 2) gai_launch_error(__FILE__, __LINE__, "act_mul: act 0 (silu), 1 (squared ReLU) or 2 (tanh cap)");
-  if (act == 2 && !(cap > 0.f)) gai_launch_error(__FILE__, __LINE__, "act_mul: the tanh cap must be positive");
+  if (act < 0 || act > 4)
+    gai_launch_error(__FILE__, __LINE__, "act_mul: act 0 (silu), 1 (squared ReLU), 2 (tanh cap), 3 (tanh GELU) or 4 (clamped gate)");
+  if ((act == 2 || act == 4) && !(cap > 0.f)) gai_launch_error(__FILE__, __LINE__, "act_mul: the cap / limit must be positive");
+  if (act == 4 && !b) gai_launch_error(__FILE__, __LINE__, "act_mul: the clamped gated activation takes two operands");
   // four elements per thread where rows, strides and base addresses allow aligned vector accesses
   const size_t esz = dt_in ? 4 : 2;
   const bool v4 = C % 4 == 0 && lda % 4 == 0 && (!b || ldb % 4 == 0) && (uintptr_t)a % (4 * esz) == 0 &&

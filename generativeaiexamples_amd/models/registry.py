@@ -19,6 +19,7 @@ from .opt import OPTConfig, OPTModel
 from .pinavik import PinavikConfig, PinavikModel
 from .ronavik import RonavikConfig, RonavikModel
 from .qwen3_next import Qwen3NextConfig, Qwen3NextModel
+from .vipolix import VipolixConfig, VipolixModel
 
 LLM_PRESETS = {
     "llama3-8b": ("meta/llama3-8b-instruct", lambda: LlamaConfig.llama3_8b()),
@@ -48,6 +49,10 @@ LLM_PRESETS = {
     # routed + identity + shared experts, looped block)
     "tiny-lituvik": ("tiny-lituvik", lambda: LituvikConfig.tiny()),
     "lituvik-1b": ("lituvik-1b", lambda: LituvikConfig.sized(2048, 18, 5632, 16, 128)),
+    # hybrid of gated linear attention and chunk-local attention beside a generalised delta rule (token shift, grouped
+    # sigmoid routing over clamped gated experts, per-layer token input)
+    "tiny-vipolix": ("tiny-vipolix", lambda: VipolixConfig.tiny()),
+    "vipolix-1b": ("vipolix-1b", lambda: VipolixConfig.sized(2048, 12, 5632, 16, 128)),
     "opt-125m": ("facebook/opt-125m", lambda: OPTConfig.opt_125m()),
     "mixtral-8x7b": ("mistralai/mixtral-8x7b-instruct-v0.1", lambda: MixtralConfig.mixtral_8x7b()),
     "tiny-moe": ("tiny-moe", lambda: MixtralConfig.tiny_moe()),
@@ -91,6 +96,8 @@ def build_llm(preset: str = "llama3-8b", weights: Optional[str] = None, device=N
             m = RonavikModel(RonavikConfig.from_json(weights), device=device, dtype=dtype or torch.bfloat16)
         elif arch == "lituvik":
             m = LituvikModel(LituvikConfig.from_json(weights), device=device, dtype=dtype or torch.bfloat16)
+        elif arch == "vipolix":
+            m = VipolixModel(VipolixConfig.from_json(weights), device=device, dtype=dtype or torch.bfloat16)
         elif arch == "opt":
             m = OPTModel(OPTConfig.from_hf(weights), device=device)
         elif arch == "mixtral":
@@ -130,6 +137,9 @@ def build_llm(preset: str = "llama3-8b", weights: Optional[str] = None, device=N
         vocab = cfg.vocab_size
     elif isinstance(cfg, LituvikConfig):
         m = LituvikModel(cfg, device=device, dtype=dtype or torch.bfloat16).random_init(seed)
+        vocab = cfg.vocab_size
+    elif isinstance(cfg, VipolixConfig):
+        m = VipolixModel(cfg, device=device, dtype=dtype or torch.bfloat16).random_init(seed)
         vocab = cfg.vocab_size
     else:
         m = LlamaModel(cfg, device=device).random_init(seed)

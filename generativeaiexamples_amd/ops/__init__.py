@@ -827,13 +827,30 @@ def decode_advance(toks, ids, pos, ctx, slots, block_tables, n_valid):
 
 
 def moe_route(logits: torch.Tensor, k: int, renorm: bool = True, score: str = "softmax", bias=None,
-              eps: float = 0.0):
+              eps: float = 0.0, groups: Optional[Sequence[int]] = None, scale: float = 1.0):
     """Router scores + top-k -> (expert ids int32 [T,k], weights fp32 [T,k]). score "softmax" (weights optionally
     renormalised over the chosen experts) or "sigmoid" (each expert scored alone; weights are the chosen scores).
     bias (fp32 [E], softmax scoring): the experts are chosen by score + bias while the weights stay the plain scores;
-    eps is added to the sum that renormalises them."""
+    eps is added to the sum that renormalises them. Sigmoid scoring with bias, groups or scale: the choice is made on
+    sigmoid score + bias; groups = (count, keep) cuts the experts into `count` equal groups of neighbours, scores a
+    group by the sum of its two largest choice scores and lets only experts of the `keep` best groups be chosen; the
+    weights are the chosen plain scores over their sum (+ eps), times scale."""
     if score not in ("softmax", "sigmoid"):
         raise ValueError(f"moe_route: unknown score function {score!r}")
+    if score == "sigmoid" and (bias is not None or groups is not None or scale != 1.0 or eps):
+        ng, keep = (int(groups[0]), int(groups[1])) if groups is not None else (1, 1)
+        E = logits.shape[1]
+        if ng < 1 or E % ng or not 1 <= keep <= ng or ng > 64:
+            raise ValueError("moe_route: groups = (count, keep) with experts % count == 0, 1 <= keep <= count <= 64")
+        if k > min(16, E // ng * keep):
+            raise ValueError("moe_route: top-k above 16 or above the experts of the kept groups")
+        if not logits.is_cuda:
+            return ref.moe_route_grouped(logits, k, bias, eps, ng, keep, scale)
+        T = logits.shape[0]
+        ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+        w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+        native().moe_route_grouped(logits.float().contiguous(), k, ids, w, bias, float(eps), ng, keep, float(scale))
+        return ids, w
     if bias is not None and score != "softmax":
         raise ValueError("moe_route: a choice bias goes with softmax scoring")
     if not logits.is_cuda:
@@ -959,21 +976,25 @@ def ep_combine(back, ids, pos, offs, w, residual, e_local: int, capacity: int):
     return out
 
 
-_MOE_ACT = {None: 0, "swiglu": 1, "relu2": 2}
+_MOE_ACT = {None: 0, "swiglu": 1, "relu2": 2, "clamp_glu": 3}
 
 
-def moe_gemm(A, a_rows, W, offs, rows_total: int, swiglu: bool = False, act: Optional[str] = None):
+def moe_gemm(A, a_rows, W, offs, rows_total: int, swiglu: bool = False, act: Optional[str] = None,
+             act_param: float = 0.0):
     """Grouped expert GEMM over expert-sorted rows (A rows gathered through a_rows when given). act: None, "swiglu"
-    (W rows interleaved [gate16 | up16]) or "relu2" (squared ReLU). bf16 operands with K % 64 == 0 run on the MFMA
+    (W rows interleaved [gate16 | up16]), "relu2" (squared ReLU) or "clamp_glu" (same interleave; g = min(gate,
+    act_param), u = clamp(up, +-act_param), g * sigmoid(1.702 g) * (u + 1)). bf16 operands with K % 64 == 0 run on the MFMA
     tiles; fp32 operands and other shapes on the generic grouped kernel (true fp32 arithmetic). offs may list more
     groups than W has experts: rows past offs[E] belong to experts without weights and are left untouched."""
     act = "swiglu" if swiglu else act
     if not A.is_cuda:
+        if act == "clamp_glu":
+            return ref.moe_gemm_clamp_glu(A, a_rows, W, offs, rows_total, act_param)
         return ref.moe_gemm(A, a_rows, W, offs, rows_total, True) if act == "swiglu" else \
             ref.moe_gemm_act(A, a_rows, W, offs, rows_total, act)
     N = W.shape[1]
-    C = torch.empty(rows_total, N // 2 if act == "swiglu" else N, dtype=A.dtype, device=A.device)
-    native().moe_gemm(A.contiguous(), a_rows, W, C, offs, rows_total, _MOE_ACT[act])
+    C = torch.empty(rows_total, N // 2 if act in ("swiglu", "clamp_glu") else N, dtype=A.dtype, device=A.device)
+    native().moe_gemm(A.contiguous(), a_rows, W, C, offs, rows_total, _MOE_ACT[act], float(act_param))
     return C
 
 
@@ -988,18 +1009,19 @@ def moe_scale_rows(h, pos, w):
     return out
 
 
-def moe_combine(Y, pos, w, residual=None, ids=None, n_real: int = 0, identity=None):
+def moe_combine(Y, pos, w, residual=None, ids=None, n_real: int = 0, identity=None, residual_gate=None):
     """out[t] = sum_j w[t, j] * Y[pos[t, j]] (+ residual); w None: plain sum (the weights were applied upstream).
+    residual_gate ([T] or a [T, 1] column slice of a wider row): the residual row is multiplied by sigmoid of it.
     With ids / n_real / identity: a chosen expert id >= n_real is an identity expert whose output is the token's own
     row identity[t] (its row of Y is not read)."""
     if not pos.is_cuda:
         if ids is not None:
             return ref.moe_combine_identity(Y, pos, w, residual, ids, n_real, identity)
-        return ref.moe_combine(Y, pos, w, residual)
+        return ref.moe_combine(Y, pos, w, residual, residual_gate)
     D = identity.shape[1] if identity is not None else Y.shape[1]
     dt = identity.dtype if identity is not None else Y.dtype
     out = torch.empty(pos.shape[0], D, dtype=dt, device=pos.device)
-    native().moe_combine(Y, pos, w, residual, out, ids, int(n_real), identity)
+    native().moe_combine(Y, pos, w, residual, out, ids, int(n_real), identity, residual_gate)
     return out
 
 
@@ -1097,11 +1119,11 @@ def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
     return y
 
 
-def gated_norm_add_f32(res: torch.Tensor, y: torch.Tensor, gate: torch.Tensor, wpost: torch.Tensor, eps: float,
+def gated_norm_add_f32(res: torch.Tensor, y: torch.Tensor, gate: Optional[torch.Tensor], wpost: torch.Tensor, eps: float,
                        wnext: Optional[torch.Tensor] = None, out_dtype=None):
     """Post-norm gated residual: fp32 ``res`` (in place) += rmsnorm(y * sigmoid(gate)) * wpost, then (out_dtype given)
     rmsnorm(res) * wnext -- or res itself when wnext is None -- in out_dtype: the closing norm of one sublayer and the
-    opening norm of the next in one pass. y / gate may be column slices of wider rows."""
+    opening norm of the next in one pass. y / gate may be column slices of wider rows; gate None: no gate."""
     if not res.is_cuda:
         return ref.gated_norm_add_f32(res, y, gate, wpost, eps, wnext, out_dtype)
     out = torch.empty(res.shape, dtype=out_dtype, device=res.device) if out_dtype is not None else None
@@ -1119,13 +1141,14 @@ def gate_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: i
     return out
 
 
-def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, nw: torch.Tensor, act: str, eps: float, out_dtype):
-    """Per-head RMS norm of fp32 o [T, H, DV], times nw ([H * DV] or shared [DV]), times silu / sigmoid of gate."""
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, nw: torch.Tensor, act: str, eps: float, out_dtype, out=None):
+    """Per-head RMS norm of fp32 o [T, H, DV], times nw ([H * DV] or shared [DV]), times silu / sigmoid of gate.
+    `out` may be a column slice of a wider buffer."""
     a = {"silu": 0, "sigmoid": 1}[act]
     if not o.is_cuda:
-        return ref.head_norm_gate(o, gate, nw, a, eps, out_dtype)
+        return _into(out, ref.head_norm_gate(o, gate, nw, a, eps, out_dtype))
     T, H, DV = o.shape
-    y = torch.empty(T, H * DV, dtype=out_dtype, device=o.device)
+    y = torch.empty(T, H * DV, dtype=out_dtype, device=o.device) if out is None else out
     native().head_norm_gate(o, gate, nw, a, float(eps), y)
     return y
 
@@ -1153,19 +1176,30 @@ def qknorm_kv_write(q, k, v, wq, wk, slots, k_cache, v_cache, H: int, G: int, DK
 
 
 def window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H: int, G: int, DK: int, DV: int, scale: float,
-                     softcap: float = 0.0, window: int = 0, r1=None, r2=None, gate=None):
-    """Sliding-window paged attention, scores capped by softcap * tanh(s / softcap) and lowered by
-    r1_h ln(1 + r2_h distance); output [T, H * DV], times sigmoid(gate) when given."""
+                     softcap: float = 0.0, window: int = 0, r1=None, r2=None, gate=None, chunk: int = 0, head_scale=None,
+                     sink: Optional[float] = None, out=None, out_scale: float = 1.0):
+    """Paged softmax attention over the visible keys j <= i: the last `window` ones (window > 0), those of the query's
+    own chunk of positions, floor(j / chunk) == floor(i / chunk) (chunk > 0), or all. Scores are capped by softcap *
+    tanh(s / softcap) and lowered by r1_h ln(1 + r2_h distance); head_scale (fp32 [H]) multiplies the scores of a head;
+    sink (a score) adds exp(sink) to the softmax denominator without a value (sink = 0: one is added). Output
+    [T, H * DV] times out_scale, times sigmoid(gate) when given (`out` may be a column slice of a wider buffer)."""
     if not q.is_cuda:
-        return ref.window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H, G, DK, DV, scale, softcap, window,
-                                    r1, r2, gate)
-    out = torch.empty(q.shape[0], H * DV, dtype=q.dtype, device=q.device)
+        if chunk or head_scale is not None or sink is not None or out_scale != 1.0:
+            if softcap or r1 is not None or gate is not None:
+                raise ValueError("window_attention: chunks, head scales and sinks go without cap, distance term and gate")
+            return _into(out, ref.masked_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H, G, DK, DV, scale,
+                                                   int(window or 0), int(chunk or 0), head_scale, sink, out_scale))
+        return _into(out, ref.window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H, G, DK, DV, scale,
+                                               softcap, window, r1, r2, gate))
+    if out is None:
+        out = torch.empty(q.shape[0], H * DV, dtype=q.dtype, device=q.device)
     # decode steps of few rows: the keys of a row are split over several waves, merged from (sums, maximum, denominator)
     T, S = q.shape[0], ctx.numel()
     ns = native().sigmoid_attention_splits(T, S, H)
     part = torch.empty(ns * T * H * (DV + 2), dtype=torch.float32, device=q.device) if ns > 1 else None
     native().window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, out, H, G, DK, DV, float(scale),
-                              float(softcap or 0.0), int(window or 0), r1, r2, gate, None, False, 1.0, part)
+                              float(softcap or 0.0), int(window or 0), r1, r2, gate, None, False, float(out_scale), part,
+                              int(chunk or 0), head_scale, None if sink is None else float(sink))
     return out
 
 
@@ -1186,7 +1220,7 @@ def sigmoid_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H: int, G: i
     ns = native().sigmoid_attention_splits(T, S, H)
     part = torch.empty(ns * T * H * DV, dtype=torch.float32, device=q.device) if ns > 1 else None
     native().window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, out, H, G, DK, DV, float(scale), 0.0,
-                              int(window or 0), None, None, None, bias, True, float(out_scale), part)
+                              int(window or 0), None, None, None, bias, True, float(out_scale), part, 0, None, None)
     return out
 
 
@@ -1327,12 +1361,13 @@ def add_dyt_f32(res: torch.Tensor, delta: Optional[torch.Tensor], extra: Optiona
     return out
 
 
-_ACT_MUL = {"silu": 0, "relu2": 1, "tanh_cap": 2}
+_ACT_MUL = {"silu": 0, "relu2": 1, "tanh_cap": 2, "gelu_tanh": 3, "clamp_glu": 4}
 
 
 def act_mul(a: torch.Tensor, b: Optional[torch.Tensor] = None, act: str = "silu", out_dtype=None, cap: float = 0.0):
-    """act(a) (* b) element by element in fp32: "silu", "relu2" (squared ReLU), "tanh_cap" (cap * tanh(a / cap)).
-    a / b may be column slices of wider rows; the result is contiguous in out_dtype (default: a's)."""
+    """act(a) (* b) element by element in fp32: "silu", "relu2" (squared ReLU), "tanh_cap" (cap * tanh(a / cap)),
+    "gelu_tanh"; "clamp_glu": the clamped gated activation min(a, cap) * sigmoid(1.702 min(a, cap)) * (clamp(b, +-cap)
+    + 1). a / b may be column slices of wider rows; the result is contiguous in out_dtype (default: a's)."""
     if act not in _ACT_MUL:
         raise ValueError(f"act_mul: unknown activation {act!r}")
     od = out_dtype or a.dtype
@@ -1385,4 +1420,62 @@ def selective_scan(x, dt, dt_bias, A, B, C, D, z, state, cu, slots, out_dtype):
         return ref.selective_scan(x, dt, dt_bias, A, B, C, D, z, state, cu, slots, out_dtype)
     out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
     native().selective_scan(x, dt, dt_bias, A, B, C, D, z, state, cu, slots, out)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# pair-interleaved partial rotation, gates and unit keys of linear recurrences, diagonal-plus-rank-one scan
+# ---------------------------------------------------------------------------------------------
+def rotary_kv_write(q, k, v, positions, slots, k_cache, v_cache, H: int, G: int, DK: int, DV: int, rot_dims: int,
+                    base: float):
+    """Rotation of the channel pairs (2i, 2i + 1), i < rot_dims / 2, of every q and k head by position *
+    base^(-2i / rot_dims) (the channels past rot_dims pass unchanged; angles in fp32 from a reduced argument), k and v
+    into their cache slots; returns the rotated q [T, H * DK] in the cache dtype. q / k / v (fp32 or the cache dtype)
+    may be column slices of one buffer."""
+    if rot_dims % 2 or not 0 <= rot_dims <= DK:
+        raise ValueError("rotary_kv_write: the rotation covers an even number of a head's channels")
+    if not q.is_cuda:
+        return ref.rotary_kv_write(q, k, v, positions, slots, k_cache, v_cache, H, G, DK, DV, rot_dims, base)
+    q_out = torch.empty(q.shape[0], H * DK, dtype=k_cache.dtype, device=q.device)
+    native().rotary_kv_write(q, k, v, positions, slots, q_out, k_cache, v_cache, H, G, DK, DV, int(rot_dims), float(base))
+    return q_out
+
+
+_DECAY_GATE = {"sigmoid": 0, "sigmoid_root": 1, "exp_sigmoid": 2}
+
+
+def decay_gate(z, bias, kind: str, param: float = 1.0):
+    """fp32 gates of a recurrence from their logits z [T, C] (+ bias [C]): "sigmoid" -> sigmoid(x); "sigmoid_root" ->
+    sigmoid(x)^(1 / param) (through its logarithm); "exp_sigmoid" -> exp(-param * sigmoid(x)). z may be a column slice."""
+    if kind not in _DECAY_GATE:
+        raise ValueError(f"decay_gate: unknown kind {kind!r}")
+    if not z.is_cuda:
+        return ref.decay_gate(z, bias, kind, param)
+    out = torch.empty(z.shape, dtype=torch.float32, device=z.device)
+    native().decay_gate(z, bias, _DECAY_GATE[kind], float(param), out)
+    return out
+
+
+def unit_key_removal(k, a, a_bias, H: int, DK: int, eps: float):
+    """Per head the unit key u = k / sqrt(sum(k^2) + eps) and the removal vector sigmoid(a + a_bias) * u: the two
+    vectors of the rank-one term of dplr_scan, fp32 [T, H * DK] each. k / a may be column slices."""
+    if not k.is_cuda:
+        return ref.unit_key_removal(k, a, a_bias, H, DK, eps)
+    av = torch.empty(k.shape[0], H * DK, dtype=torch.float32, device=k.device)
+    bv = torch.empty_like(av)
+    native().unit_key_removal(k, a, a_bias, H, DK, float(eps), av, bv)
+    return av, bv
+
+
+def dplr_scan(q, k, v, decay, av, bv, state, cu, slots, q_scale: float = 1.0):
+    """Linear recurrence with a diagonal decay plus a rank-one removal, per head:
+    S_t = diag(decay_t) S_(t-1) - av_t (bv_t^T S_(t-1)) + k_t v_t^T,  o_t = q_scale * S_t^T q_t
+    (both terms read the old state; av / bv None: gated linear attention). q / k [T, H * DK] and v [T, H * DV] in the
+    activation dtype (column slices of a projection), decay / av / bv fp32 [T, H * DK]; state [slots, H, DK, DV] fp32 in
+    place -> fp32 [T, H, DV]."""
+    if not q.is_cuda:
+        return ref.dplr_scan(q, k, v, decay, av, bv, state, cu, slots, q_scale)
+    H, DV = state.shape[1], state.shape[3]
+    out = torch.empty(q.shape[0], H, DV, dtype=torch.float32, device=q.device)
+    native().dplr_scan(q, k, v, decay, av, bv, state, cu, slots, out, float(q_scale))
     return out

@@ -274,11 +274,12 @@ def moe_gemm(A, a_rows, W, offs, rows_total, swiglu):
     return C
 
 
-def moe_combine(Y, pos, w, residual=None):
+def moe_combine(Y, pos, w, residual=None, residual_gate=None):
     y = Y[pos.long()].float()
     y = (y * w.float()[..., None]).sum(1) if w is not None else y.sum(1)
     if residual is not None:
-        y = y + residual.float()
+        r = residual.float()
+        y = y + (r * torch.sigmoid(residual_gate.float().reshape(-1, 1)) if residual_gate is not None else r)
     return y.to(Y.dtype)
 
 
@@ -613,7 +614,7 @@ def embed_pos_f32(ids, table, scale, positions, pos_table):
 def gated_norm_add_f32(res, y, gate, wpost, eps, wnext, out_dtype):
     """res (fp32, in place) += rmsnorm(y * sigmoid(gate)) * wpost; returns rmsnorm(res) * wnext (wnext None: res) as
     out_dtype, or None when out_dtype is None."""
-    g = y.float() * torch.sigmoid(gate.float())
+    g = y.float() * torch.sigmoid(gate.float()) if gate is not None else y.float()
     res.add_(g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps) * wpost.float())
     return add_rmsnorm_f32(res, None, 1.0, wnext, eps, out_dtype)
 
@@ -767,9 +768,14 @@ def add_dyt_f32(res, delta, extra, alpha, w, b, out_dtype):
 
 
 def act_mul(a, b, act, out_dtype, cap=0.0):
-    """act(a) (* b): "silu", "relu2" (squared ReLU) or "tanh_cap" (cap tanh(a / cap)), in fp32."""
+    """act(a) (* b): "silu", "relu2" (squared ReLU), "tanh_cap" (cap tanh(a / cap)), "gelu_tanh", or "clamp_glu" (the
+    clamped gated activation of a, b with limit cap), in fp32."""
     x = a.float()
-    if act == "silu":
+    if act == "clamp_glu":
+        return clamp_glu(x, b, cap).to(out_dtype)
+    if act == "gelu_tanh":
+        y = F.gelu(x, approximate="tanh")
+    elif act == "silu":
         y = F.silu(x)
     elif act == "relu2":
         y = torch.relu(x) ** 2
@@ -883,3 +889,155 @@ def moe_combine_identity(Y, pos, w, residual, ids, n_real, h):
     if residual is not None:
         out = out + residual.float()
     return out.to(h.dtype)
+
+
+# ---------------------------------------------------------------------------------------------
+# pair-interleaved partial rotation, chunk-local attention with a sink and per-head temperatures, diagonal-plus-rank-one
+# linear recurrences (gated linear attention, generalised delta rule), group-limited sigmoid routing, clamped gated
+# experts
+# ---------------------------------------------------------------------------------------------
+GLU_SLOPE = 1.702      # slope of the sigmoid in the clamped gated activation
+
+
+def rotary_kv_write(q, k, v, positions, slots, k_cache, v_cache, H, G, DK, DV, rot_dims, base):
+    """Rotation of the channel pairs (2i, 2i + 1), i < rot_dims / 2, of every q and k head by position * base^(-2i /
+    rot_dims) (channels past rot_dims pass unchanged); k and v into their cache slots; returns q [T, H * DK]."""
+    T = q.shape[0]
+    pos = positions[:T].to(torch.float64)
+
+    def rot(x):
+        x = x.float()
+        if not rot_dims:
+            return x
+        i = torch.arange(rot_dims // 2, dtype=torch.float64)
+        ang = pos[:, None] * float(base) ** (-2.0 * i / rot_dims)
+        c, s = torch.cos(ang).float()[:, None, :], torch.sin(ang).float()[:, None, :]
+        a, b = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+        y = x.clone()
+        y[..., 0:rot_dims:2] = a * c - b * s
+        y[..., 1:rot_dims:2] = b * c + a * s
+        return y
+
+    s = slots[:T].long()
+    k_cache[s // BLOCK, :, s % BLOCK] = rot(k.reshape(T, G, DK)).to(k_cache.dtype)
+    v_cache[s // BLOCK, :, :, s % BLOCK] = v.reshape(T, G, DV).to(v_cache.dtype)
+    return rot(q.reshape(T, H, DK)).reshape(T, H * DK).to(k_cache.dtype)
+
+
+def masked_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H, G, DK, DV, scale, window, chunk, head_scale, sink,
+                     out_scale):
+    """Softmax attention over the visible keys j <= i: the last `window` ones (window > 0), those of the query's own
+    chunk of positions floor(i / chunk) = floor(j / chunk) (chunk > 0), or all. head_scale [H] multiplies the scores of
+    a head; sink (a score, or None) adds exp(sink) to the softmax denominator without adding a value."""
+    T = q.numel() // (H * DK)
+    q3 = q.float().view(T, H, DK)
+    out = torch.zeros(T, H, DV)
+    cu = [int(x) for x in cu_q.tolist()]
+    for s, n in enumerate(ctx.tolist()):
+        b, e = cu[s], cu[s + 1]
+        if e <= b:
+            continue
+        n = int(n)
+        pages = block_tables[s, : (n + BLOCK - 1) // BLOCK].long()
+        K = k_cache[pages].float().permute(1, 0, 2, 3).reshape(G, -1, DK)[:, :n]
+        V = v_cache[pages].float().permute(1, 0, 3, 2).reshape(G, -1, DV)[:, :n]
+        pos = torch.arange(n - (e - b), n)
+        key = torch.arange(n)
+        vis = key[None, :] <= pos[:, None]
+        if window > 0:
+            vis = vis & (pos[:, None] - key[None, :] < window)
+        if chunk > 0:
+            vis = vis & (torch.div(pos, chunk, rounding_mode="floor")[:, None] ==
+                         torch.div(key, chunk, rounding_mode="floor")[None, :])
+        for h in range(H):
+            sc = (q3[b:e, h] @ K[h // (H // G)].t()) * (scale * (float(head_scale[h]) if head_scale is not None else 1.0))
+            sc = sc.masked_fill(~vis, float("-inf"))
+            m = sc.max(-1, keepdim=True).values
+            if sink is not None:
+                m = m.clamp(min=float(sink))
+            p = torch.exp(sc - m)
+            den = p.sum(-1, keepdim=True)
+            if sink is not None:
+                den = den + torch.exp(float(sink) - m)
+            out[b:e, h] = (p / den) @ V[h // (H // G)]
+    return (out.reshape(T, H * DV) * float(out_scale)).to(q.dtype)
+
+
+def decay_gate(z, bias, kind, param):
+    """fp32 gates of a recurrence from their logits z (+ bias): "sigmoid" -> sigmoid(x); "sigmoid_root" ->
+    sigmoid(x)^(1 / param); "exp_sigmoid" -> exp(-param * sigmoid(x))."""
+    x = z.float() + (bias.float().reshape(1, -1) if bias is not None else 0.0)
+    if kind == "sigmoid":
+        return torch.sigmoid(x)
+    if kind == "sigmoid_root":
+        return torch.exp(F.logsigmoid(x) / float(param))
+    return torch.exp(-float(param) * torch.sigmoid(x))
+
+
+def unit_key_removal(k, a, a_bias, H, DK, eps):
+    """Per head the unit key u = k / sqrt(sum(k^2) + eps) and the removal vector sigmoid(a + a_bias) * u (both fp32
+    [T, H * DK])."""
+    T = k.shape[0]
+    k3 = k.float().reshape(T, H, DK)
+    u = k3 * torch.rsqrt(k3.pow(2).sum(-1, keepdim=True) + eps)
+    rate = torch.sigmoid(a.float() + (a_bias.float().reshape(1, -1) if a_bias is not None else 0.0)).reshape(T, H, DK)
+    return (rate * u).reshape(T, H * DK), u.reshape(T, H * DK)
+
+
+def dplr_scan(q, k, v, decay, av, bv, state, cu, slots, q_scale):
+    """S_t = diag(decay_t) S_(t-1) - av_t (bv_t^T S_(t-1)) + k_t v_t^T, o_t = q_scale * S_t^T q_t (av / bv None: no
+    removal term). q / k / decay / av / bv [T, H * DK], v [T, H * DV]; state [slots, H, DK, DV] fp32 in place."""
+    H, DK, DV = state.shape[1:]
+    T = q.shape[0]
+    r3 = lambda t: t.float().reshape(T, H, -1)  # noqa: E731
+    q3, k3, v3, w3 = r3(q), r3(k), r3(v), r3(decay)
+    a3, b3 = (r3(av), r3(bv)) if av is not None else (None, None)
+    out = torch.empty(T, H, DV)
+    for lo, hi, s in _seqs(cu, slots):
+        S = state[s]
+        for t in range(lo, hi):
+            new = w3[t][:, :, None] * S + k3[t][:, :, None] * v3[t][:, None, :]
+            if a3 is not None:
+                new = new - a3[t][:, :, None] * torch.einsum("hk,hkv->hv", b3[t], S)[:, None, :]
+            S = new
+            out[t] = torch.einsum("hkv,hk->hv", S, q3[t]) * float(q_scale)
+        if hi > lo:
+            state[s] = S
+    return out
+
+
+def moe_route_grouped(logits, k, bias, eps, groups, keep, scale, group_top=2):
+    """Sigmoid scores s; choice scores s + bias; the experts form `groups` equal groups of neighbours, a group scores
+    the sum of its group_top largest choice scores and only experts of the `keep` best groups can be chosen; weights
+    s / (sum of the chosen s + eps) * scale."""
+    s = torch.sigmoid(logits.float())
+    c = s + bias.float() if bias is not None else s.clone()
+    T, E = c.shape
+    if groups > 1 and keep < groups:
+        per = c.view(T, groups, E // groups)
+        gs = per.topk(min(group_top, E // groups), -1).values.sum(-1)
+        best = gs.topk(keep, -1).indices
+        ok = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, best, True)
+        c = torch.where(ok[:, :, None].expand_as(per).reshape(T, E), c, torch.full_like(c, float("-inf")))
+    ids = torch.topk(c, k, dim=-1).indices
+    w = torch.gather(s, 1, ids)
+    return ids.int(), w / (w.sum(-1, keepdim=True) + eps) * float(scale)
+
+
+def clamp_glu(g, u, limit):
+    g = g.float().clamp(max=float(limit))
+    u = u.float().clamp(-float(limit), float(limit))
+    return g * torch.sigmoid(GLU_SLOPE * g) * (u + 1.0)
+
+
+def moe_gemm_clamp_glu(A, a_rows, W, offs, rows_total, limit):
+    """Grouped GEMM whose rows of W are interleaved [gate16 | up16] blocks, with the clamped gated activation."""
+    E, N, K = W.shape
+    C = torch.empty(rows_total, N // 2, dtype=A.dtype)
+    o = offs.tolist()
+    for e in range(E):
+        if o[e + 1] > o[e]:
+            rows = A[a_rows[o[e]:o[e + 1]].long()] if a_rows is not None else A[o[e]:o[e + 1]]
+            y = (rows.float() @ W[e].float().t()).view(rows.shape[0], N // 32, 2, 16)
+            C[o[e]:o[e + 1]] = clamp_glu(y[:, :, 0], y[:, :, 1], limit).reshape(rows.shape[0], N // 2).to(A.dtype)
+    return C
