@@ -21,6 +21,12 @@
 //                     dt_c = softplus(dt + dt_bias); S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n;
 //                     y_c = sum_n S[c, n] C_n + D_c x_c; out = y * silu(z)
 //
+//   decay_gate        token-parallel fp32 gates of a recurrence from their logits: sigmoid(x), sigmoid(x)^(1 / p) (through
+//                     its logarithm -softplus(-x) / p) or exp(-p sigmoid(x))
+//   unit_key_removal  per head the unit key u = k / sqrt(sum k^2 + eps) and the removal vector sigmoid(a + bias) * u
+//   dplr_scan         diagonal decay plus a rank-one removal: S <- diag(w_t) S - av_t (bv_t^T S) + k_t v_t^T (both terms
+//                     read the old state), o_t = scale * S^T q_t; without av / bv it is gated linear attention
+//
 // A batch is S sequences of rows [cu[s], cu[s+1]) with pool slot slots[s] (device vectors: graph-capturable); a decoded
 // token is a sequence of one row, a prompt portion a longer one. The scans keep the state in VGPRs for the whole
 // portion and read / write the pool once. Two shapes per recurrence:
@@ -499,6 +505,244 @@ __global__ __launch_bounds__(64) void delta_scan_cols_kernel(const float* __rest
       }
       const float oo = rowgroup_sum<RGS>(o0 + o1);
       if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * DV + j] = oo;
+    }
+  }
+  if (on) {
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (i < nrow) Sg[(size_t)i * DV] = col[i];
+  }
+}
+
+// ---- diagonal decay plus rank-one removal (gated linear attention, generalised delta rule) --------------------------
+// The two shapes of delta_scan: decode steps with one workgroup per (head, sequence) and coalesced state streaming,
+// prompt portions with one wave64 per block of state columns. q / k / v come in the activation dtype (column slices of
+// a projection output), decay and the removal vectors in fp32; all arithmetic fp32.
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+template <typename TA>
+__global__ __launch_bounds__(256) void decay_gate_kernel(const TA* __restrict__ z, int ldz, const float* __restrict__ bias,
+                                                         int kind, float param, float* __restrict__ out, int T, int C) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long)T * C) return;
+  const int t = (int)(e / C), c = (int)(e % C);
+  const float x = (float)z[(size_t)t * ldz + c] + (bias ? bias[c] : 0.f);
+  float y;
+  if (kind == 0) y = sigmoid_f(x);
+  else if (kind == 1) {  // sigmoid(x)^(1 / param) = exp(-softplus(-x) / param)
+    const float sp = -x > 20.f ? -x : log1pf(expf(-x));
+    y = expf(-sp / param);
+  } else y = expf(-param * sigmoid_f(x));
+  out[e] = y;
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void unit_key_removal_kernel(const TA* __restrict__ k, int ldk, const TA* __restrict__ a,
+                                                               int lda, const float* __restrict__ a_bias,
+                                                               float* __restrict__ av, float* __restrict__ bv, int TH,
+                                                               int H, int DK, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int th = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (th >= TH) return;
+  const int t = th / H, h = th - t * H;
+  const TA* kr = k + (size_t)t * ldk + (size_t)h * DK;
+  const TA* ar = a + (size_t)t * lda + (size_t)h * DK;
+  float ss = 0.f;
+  for (int i = lane; i < DK; i += 64) {
+    const float x = (float)kr[i];
+    ss += x * x;
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss + eps);
+  for (int i = lane; i < DK; i += 64) {
+    const float u = (float)kr[i] * inv;
+    const float rate = sigmoid_f((float)ar[i] + (a_bias ? a_bias[(size_t)h * DK + i] : 0.f));
+    bv[(size_t)th * DK + i] = u;
+    av[(size_t)th * DK + i] = rate * u;
+  }
+}
+
+template <typename TA, bool RANK1>
+__global__ __launch_bounds__(1024) void dplr_scan_kernel(const TA* __restrict__ q, int ldq, const TA* __restrict__ k, int ldk,
+                                                         const TA* __restrict__ v, int ldv, const float* __restrict__ decay,
+                                                         const float* __restrict__ av, const float* __restrict__ bv,
+                                                         float* __restrict__ state, const int* __restrict__ cu,
+                                                         const int* __restrict__ slots, float* __restrict__ out, int H,
+                                                         int DK, int DV, float q_scale) {
+  extern __shared__ float lds[];  // buf[2][5][DK] (q, k, w, a, b) | red[2][2][RG][DV]
+  const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
+  const int RG = (DK + kRows - 1) / kRows;
+  const int j = tid % DV, rg = tid / DV;
+  const int row0 = rg * kRows, nrow = min(kRows, DK - row0);
+  float* buf = lds;
+  float* red = buf + 10 * DK;
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  float* Sg = state + (((size_t)slots[s] * H + h) * DK + row0) * DV + j;
+  float col[kRows];
+#pragma unroll
+  for (int i = 0; i < kRows; ++i) col[i] = i < nrow ? Sg[(size_t)i * DV] : 0.f;
+  for (int t = t0; t < t1; ++t) {
+    const int b = (t - t0) & 1;
+    float* qb = buf + b * 5 * DK;
+    for (int i = tid; i < DK; i += blockDim.x) {
+      const size_t o = ((size_t)t * H + h) * DK + i;
+      qb[i] = (float)q[(size_t)t * ldq + (size_t)h * DK + i];
+      qb[DK + i] = (float)k[(size_t)t * ldk + (size_t)h * DK + i];
+      qb[2 * DK + i] = decay[o];
+      if (RANK1) {
+        qb[3 * DK + i] = av[o];
+        qb[4 * DK + i] = bv[o];
+      }
+    }
+    const float vj = (float)v[(size_t)t * ldv + (size_t)h * DV + j];
+    __syncthreads();
+    float mm = 0.f;
+    if (RANK1) {
+#pragma unroll
+      for (int i = 0; i < kRows; ++i)
+        if (i < nrow) mm = fmaf(col[i], qb[4 * DK + row0 + i], mm);
+      if (RG > 1) {
+        float* rm = red + ((b * 2 + 0) * RG) * DV;
+        rm[rg * DV + j] = mm;
+        __syncthreads();
+        mm = 0.f;
+        for (int x = 0; x < RG; ++x) mm += rm[x * DV + j];
+      }
+    }
+    float oo = 0.f;
+#pragma unroll
+    for (int i = 0; i < kRows; ++i) {
+      if (i < nrow) {
+        float c = fmaf(qb[2 * DK + row0 + i], col[i], qb[DK + row0 + i] * vj);
+        if (RANK1) c = fmaf(-qb[3 * DK + row0 + i], mm, c);
+        col[i] = c;
+        oo = fmaf(c, qb[row0 + i], oo);
+      }
+    }
+    if (RG == 1) {
+      out[((size_t)t * H + h) * DV + j] = oo * q_scale;
+    } else {
+      float* ro = red + ((b * 2 + 1) * RG) * DV;
+      ro[rg * DV + j] = oo;
+      __syncthreads();
+      if (rg == 0) {
+        float o = 0.f;
+        for (int x = 0; x < RG; ++x) o += ro[x * DV + j];
+        out[((size_t)t * H + h) * DV + j] = o * q_scale;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kRows; ++i)
+    if (i < nrow) Sg[(size_t)i * DV] = col[i];
+}
+
+template <typename TA, int R, int RGS, bool RANK1>
+__global__ __launch_bounds__(64) void dplr_scan_cols_kernel(const TA* __restrict__ q, int ldq, const TA* __restrict__ k,
+                                                            int ldk, const TA* __restrict__ v, int ldv,
+                                                            const float* __restrict__ decay, const float* __restrict__ av,
+                                                            const float* __restrict__ bv, float* __restrict__ state,
+                                                            const int* __restrict__ cu, const int* __restrict__ slots,
+                                                            float* __restrict__ out, int H, int DK, int DV,
+                                                            float q_scale) {
+  constexpr int COLS = 64 / RGS, NP = kTB * RGS * R / 64, LD = RGS * R + RGS, NA = RANK1 ? 5 : 3;
+  extern __shared__ float lds[];
+  const int h = blockIdx.x, s = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
+  const int jj = lane / RGS, rg = lane % RGS, j = cb * COLS + jj;
+  const bool on = j < DV;
+  const int row0 = rg * R, nrow = max(0, min(R, DK - row0));
+  float* qs = lds;
+  float* ks = qs + kTB * LD;
+  float* ws = ks + kTB * LD;
+  float* as = ws + kTB * LD;     // RANK1 only
+  float* bs = as + kTB * LD;
+  float* vs = lds + NA * kTB * LD;  // [kTB][COLS]
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  for (int x = lane; x < NA * kTB * LD; x += 64) lds[x] = 0.f;
+  float* Sg = state + (((size_t)slots[s] * H + h) * DK + row0) * DV + j;
+  float col[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) col[i] = (on && i < nrow) ? Sg[(size_t)i * DV] : 0.f;
+  constexpr int NPART = 64 / kTB;
+  static_assert(NP * NPART >= RGS * R, "staging covers a full row");
+  const int stt = lane / NPART, spart = lane % NPART;
+  float pq[NP], pk[NP], pw[NP], pa[RANK1 ? NP : 1], pb[RANK1 ? NP : 1], pv[2];
+  auto fetch = [&](int tb) {
+    const int n = min(kTB, t1 - tb);
+#pragma unroll
+    for (int x = 0; x < NP; ++x) {
+      const int i = spart + NPART * x;
+      if (stt < n && i < DK) {
+        const size_t o = ((size_t)(tb + stt) * H + h) * DK + i;
+        pq[x] = (float)q[(size_t)(tb + stt) * ldq + (size_t)h * DK + i];
+        pk[x] = (float)k[(size_t)(tb + stt) * ldk + (size_t)h * DK + i];
+        pw[x] = decay[o];
+        if (RANK1) {
+          pa[x] = av[o];
+          pb[x] = bv[o];
+        }
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+      const int idx = x * 64 + lane, tt = idx / COLS, c = cb * COLS + idx % COLS;
+      pv[x] = (tt < n && c < DV) ? (float)v[(size_t)(tb + tt) * ldv + (size_t)h * DV + c] : 0.f;
+    }
+  };
+  fetch(t0);
+  for (int tb = t0; tb < t1; tb += kTB) {
+    const int n = min(kTB, t1 - tb);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int x = 0; x < NP; ++x) {
+      const int i = spart + NPART * x;
+      if (stt < n && i < DK) {
+        const int a = stt * LD + lds_row<R>(i);
+        qs[a] = pq[x];
+        ks[a] = pk[x];
+        ws[a] = pw[x];
+        if (RANK1) {
+          as[a] = pa[x];
+          bs[a] = pb[x];
+        }
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+      if (x * 64 + lane < kTB * COLS) vs[x * 64 + lane] = pv[x];
+    __builtin_amdgcn_wave_barrier();
+    if (tb + kTB < t1) fetch(tb + kTB);
+    for (int tt = 0; tt < n; ++tt) {
+      const float vj = vs[tt * COLS + jj];
+      const int a = tt * LD + row0 + rg;
+      float mm = 0.f;
+      if (RANK1) {
+        float m0 = 0.f, m1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; i += 2) {
+          m0 = fmaf(col[i], bs[a + i], m0);
+          m1 = fmaf(col[i + 1], bs[a + i + 1], m1);
+        }
+        mm = rowgroup_sum<RGS>(m0 + m1);
+      }
+      float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; i += 2) {
+        float c0 = fmaf(ws[a + i], col[i], ks[a + i] * vj);
+        float c1 = fmaf(ws[a + i + 1], col[i + 1], ks[a + i + 1] * vj);
+        if (RANK1) {
+          c0 = fmaf(-as[a + i], mm, c0);
+          c1 = fmaf(-as[a + i + 1], mm, c1);
+        }
+        col[i] = c0;
+        col[i + 1] = c1;
+        o0 = fmaf(c0, qs[a + i], o0);
+        o1 = fmaf(c1, qs[a + i + 1], o1);
+      }
+      const float oo = rowgroup_sum<RGS>(o0 + o1);
+      if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * DV + j] = oo * q_scale;
     }
   }
   if (on) {
@@ -1343,6 +1587,73 @@ void gai_delta_scan(const float* q, const float* k, const float* v, int ldv, con
   const dim3 grid(H, S);
   const size_t lds = (size_t)(6 * DK + 4 * RG * DV) * sizeof(float);
   delta_scan_kernel<<<grid, DV * RG, lds, st>>>(q, k, v, ldv, decay, beta, state, cu, slots, out, H, G, DK, DV);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_decay_gate(const void* z, int ldz, const float* bias, int kind, float param, float* out, int T, int C, int dt,
+                    hipStream_t st) {
+  if (T == 0 || C == 0) return;
+  if (kind < 0 || kind > 2) gai_launch_error(__FILE__, __LINE__, "decay_gate: kind 0 (sigmoid), 1 (sigmoid root) or 2 (exp of sigmoid)");
+  if (kind == 1 && !(param > 0.f)) gai_launch_error(__FILE__, __LINE__, "decay_gate: the root must be positive");
+  const unsigned grid = (unsigned)(((long)T * C + 255) / 256);
+  if (dt)
+    decay_gate_kernel<float><<<grid, 256, 0, st>>>((const float*)z, ldz, bias, kind, param, out, T, C);
+  else
+    decay_gate_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)z, ldz, bias, kind, param, out, T, C);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_unit_key_removal(const void* k, int ldk, const void* a, int lda, const float* a_bias, float* av, float* bv, int T,
+                          int H, int DK, float eps, int dt, hipStream_t st) {
+  if (T == 0) return;
+  const int TH = T * H, grid = (TH + 3) / 4;
+  if (dt)
+    unit_key_removal_kernel<float><<<grid, 256, 0, st>>>((const float*)k, ldk, (const float*)a, lda, a_bias, av, bv, TH, H,
+                                                          DK, eps);
+  else
+    unit_key_removal_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)k, ldk, (const bf16*)a, lda, a_bias, av, bv, TH, H, DK,
+                                                         eps);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_dplr_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* decay,
+                   const float* av, const float* bv, float* state, const int* cu, const int* slots, int S, int T,
+                   float* out, int H, int DK, int DV, float q_scale, int dt, hipStream_t st) {
+  if (S == 0 || T == 0) return;
+  if (DK > kMaxDK) gai_launch_error(__FILE__, __LINE__, "dplr_scan: key head size above 256");
+  if ((av == nullptr) != (bv == nullptr)) gai_launch_error(__FILE__, __LINE__, "dplr_scan: the two removal vectors come together");
+  const bool r1 = av != nullptr;
+  if (T > S) {  // some sequence brings more than one row: the column-sliced scan
+#define GAI_DPLR_C(TA, R, RGS, R1)                                                                                   \
+  do {                                                                                                               \
+    const dim3 grid(H, S, (DV + 64 / RGS - 1) / (64 / RGS));                                                         \
+    const size_t lds = (size_t)((R1 ? 5 : 3) * kTB * (RGS * R + RGS) + kTB * (64 / RGS)) * sizeof(float);            \
+    dplr_scan_cols_kernel<TA, R, RGS, R1><<<grid, 64, lds, st>>>((const TA*)q, ldq, (const TA*)k, ldk, (const TA*)v, \
+                                                                 ldv, decay, av, bv, state, cu, slots, out, H, DK,   \
+                                                                 DV, q_scale);                                       \
+  } while (0)
+#define GAI_DPLR_S(TA, R1)                                                                                           \
+  do {                                                                                                               \
+    if (DK <= 64) GAI_DPLR_C(TA, 8, 8, R1); else if (DK <= 128) GAI_DPLR_C(TA, 8, 16, R1);                           \
+    else GAI_DPLR_C(TA, 16, 16, R1);                                                                                 \
+  } while (0)
+    if (dt) { if (r1) GAI_DPLR_S(float, true); else GAI_DPLR_S(float, false); }
+    else { if (r1) GAI_DPLR_S(bf16, true); else GAI_DPLR_S(bf16, false); }
+#undef GAI_DPLR_S
+#undef GAI_DPLR_C
+    GAI_LAUNCH_CHECK();
+    return;
+  }
+  const int RG = (DK + kRows - 1) / kRows;
+  if (DV * RG > 1024) gai_launch_error(__FILE__, __LINE__, "dplr_scan: head sizes above 256");
+  const dim3 grid(H, S);
+  const size_t lds = (size_t)(10 * DK + 4 * RG * DV) * sizeof(float);
+#define GAI_DPLR(TA, R1)                                                                                             \
+  dplr_scan_kernel<TA, R1><<<grid, DV * RG, lds, st>>>((const TA*)q, ldq, (const TA*)k, ldk, (const TA*)v, ldv, decay, \
+                                                       av, bv, state, cu, slots, out, H, DK, DV, q_scale)
+  if (dt) { if (r1) GAI_DPLR(float, true); else GAI_DPLR(float, false); }
+  else { if (r1) GAI_DPLR(bf16, true); else GAI_DPLR(bf16, false); }
+#undef GAI_DPLR
   GAI_LAUNCH_CHECK();
 }
 

@@ -249,7 +249,6 @@ class VipolixModel:
         self.pool = StatePool(state_slots or int(os.environ.get("GAI_LINEAR_STATE_SLOTS", "64")), self.device)
         self.state: Dict[int, Dict[str, torch.Tensor]] = {}
         self.capture_residuals: Optional[list] = None  # numerics debugging: the residual stream after every layer
-        self.route_all = False  # numerics debugging: every expert is chosen (no discrete decision), weights as routed
         self._i32 = dict(dtype=torch.int32, device=self.device)
 
     # ------------------------------------------------------------------ engine sizing hooks
@@ -477,9 +476,6 @@ class VipolixModel:
         g = r["groups"]
         ids, wts = ops.moe_route(logits, top, score="sigmoid", bias=w.get(q + "correction"), eps=ROUTE_EPS,
                                  groups=(g["count"], g["keep"]), scale=float(r["scale"]))
-        if self.route_all:
-            ids, wts = _all_experts(ids, wts, E)
-            top = E
         shared = sgate = None
         if ml.get("shared"):
             Fs = w[q + "shared.down"].shape[1]
@@ -533,12 +529,3 @@ class VipolixModel:
             res = res.index_select(0, fb.sample_rows)
         xf = ops.add_rmsnorm_f32(res, None, 1.0, w["final.norm"], eps, dt)
         return ops.linear(xf, w["head"], out_dtype=torch.float32)[:, : c.vocab_size]
-
-
-def _all_experts(ids, wts, E: int):
-    """Every expert listed for every token, the routed ones with their weights and the others with weight zero (the
-    same kernels run, but no discrete decision depends on rounding)."""
-    T = ids.shape[0]
-    full = torch.zeros(T, E, dtype=torch.float32, device=ids.device)
-    full.scatter_(1, ids.long(), wts)
-    return torch.arange(E, dtype=torch.int32, device=ids.device).repeat(T, 1).contiguous(), full

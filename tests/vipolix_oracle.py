@@ -200,3 +200,130 @@ def forward(cfg: dict, sd: Dict[str, torch.Tensor], tokens: List[int], residuals
         if residuals is not None:
             residuals.append(x.clone())
     return centred_norm(x, W["final.norm"], eps) @ W["head"].T
+
+
+# ------------------------------------------------------------------------------------------------ made-up checkpoints
+def gla(heads=2, dim=8, vdim=12, tau=6.0):
+    return dict(type="gla", mixer=dict(heads=heads, dim=dim, vdim=vdim, tau=tau))
+
+
+def par(heads=4, kv_heads=2, dim=8, vdim=12, conv=3, chunk=11, rot=4, base=100.0, scale=0.4, rheads=2, rdim=8,
+        left_scale=0.7, right_scale=1.3):
+    left = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, conv=conv, scale=scale, mask=dict(size=chunk),
+                rot=dict(base=base, dims=rot))
+    return dict(type="parallel", mixer=dict(left=left, right=dict(heads=rheads, dim=rdim), left_scale=left_scale,
+                                            right_scale=right_scale))
+
+
+def moe_ff(layer, ff=16, experts=6, top=2, groups=3, keep=2, scale=1.4, limit=1.5, shared=24, shared_limit=2.5):
+    ml = dict(kind="moe", expert=dict(ff=ff, limit=limit),
+              router=dict(experts=experts, top=top, scale=scale, groups=dict(count=groups, keep=keep)))
+    if shared:
+        ml["shared"] = dict(ff=shared, limit=shared_limit)
+    return dict(layer, mlp=ml)
+
+
+def no_ff(layer):
+    return dict(layer, mlp=None)
+
+
+def make_config(layers, width=32, vocab=96, side=6, eps=1e-5):
+    cfg = dict(architecture="Vipolix", layers=list(layers), norm=dict(eps=eps), vocab=vocab, width=width)
+    if side:
+        cfg["token_side"] = dict(dim=side)
+    return cfg
+
+
+def random_checkpoint(cfg, seed, slow_decay=False, low_rank=5):
+    """bf16-representable random tensors with the checkpoint's names, sized so that every mechanism matters: biases,
+    temperatures, corrections and norm weights well away from their neutral values."""
+    g = torch.Generator().manual_seed(seed)
+    D, V = cfg["width"], cfg["vocab"]
+    rn = lambda *s, std=1.0: (torch.randn(*s, generator=g) * std).bfloat16().float()  # noqa: E731
+    un = lambda *s, lo=0.0, hi=1.0: (torch.rand(*s, generator=g) * (hi - lo) + lo).bfloat16().float()  # noqa: E731
+    lin = lambda o, i, gain=1.0: rn(o, i, std=gain * i ** -0.5)  # noqa: E731
+    sd = {"embed": rn(V, D), "head": lin(V, D, 2.0), "final.norm": rn(D, std=0.3)}
+    sdim = int((cfg.get("token_side") or {}).get("dim") or 0)
+    if sdim:
+        sd["side.embed"] = rn(V, len(cfg["layers"]) * sdim)
+    for i, l in enumerate(cfg["layers"]):
+        p, x, m = f"l{i}.", f"l{i}.mix.", l["mixer"]
+        sd[p + "norm1"], sd[p + "shift"] = rn(D, std=0.3), un(D, lo=-0.2, hi=0.9)
+        if l["type"] == "gla":
+            H, dk, dv = m["heads"], m["dim"], m["vdim"]
+            sd[x + "q"], sd[x + "k"], sd[x + "v"] = lin(H * dk, D, 2.0), lin(H * dk, D), lin(H * dv, D)
+            sd[x + "g"], sd[x + "o"] = lin(H * dv, D, 1.5), lin(D, H * dv)
+            sd[x + "norm"] = 1 + rn(dv, std=0.3)
+            sd[x + "a1"], sd[x + "a2"] = lin(low_rank, D), lin(H * dk, low_rank, 2.0)
+            sd[x + "a2.b"] = un(H * dk, lo=5.0, hi=8.0) if slow_decay else un(H * dk, lo=-1.0, hi=4.0)
+        else:
+            a, r = m["left"], m["right"]
+            H, G, dk, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            xl, xr = x + "left.", x + "right."
+            for n, rows in (("q", H * dk), ("k", G * dk), ("v", G * dv)):
+                sd[xl + n], sd[xl + n + ".b"] = lin(rows, D, 1.0 if n == "v" else 2.0), rn(rows, std=0.3)
+                if a.get("conv"):
+                    sd[xl + n + ".conv"] = rn(rows, a["conv"], std=0.4)
+                    sd[xl + n + ".conv"][:, -1] += 1.0
+            sd[xl + "temp"], sd[xl + "o"] = un(H, lo=0.5, hi=1.6), lin(D, H * dv)
+            Hr, d = r["heads"], r["dim"]
+            for n in ("r", "k", "v", "g", "a"):
+                sd[xr + n] = lin(Hr * d, D, 1.5)
+            sd[xr + "a.b"] = rn(Hr * d, std=0.7)
+            sd[xr + "w1"], sd[xr + "w2"] = lin(low_rank, D, 1.5), lin(Hr * d, low_rank, 2.0)
+            sd[xr + "w0"] = un(Hr * d, lo=-9.0, hi=-6.0) if slow_decay else un(Hr * d, lo=-3.0, hi=2.0)
+            sd[xr + "norm"], sd[xr + "o"] = 1 + rn(Hr * d, std=0.3), lin(D, Hr * d)
+        ml = l.get("mlp")
+        if ml is not None:
+            sd[p + "norm2"] = rn(D, std=0.3)
+            q, r = p + "mlp.", ml["router"]
+            for e in list(range(r["experts"])) + (["shared"] if ml.get("shared") else []):
+                pre = q + (f"e{e}." if e != "shared" else "shared.")
+                F_ = ml["shared"]["ff"] if e == "shared" else ml["expert"]["ff"]
+                sd[pre + "gate"], sd[pre + "up"], sd[pre + "down"] = lin(F_, D, 2.0), lin(F_, D, 2.0), lin(D, F_)
+            sd[q + "router"], sd[q + "correction"] = lin(r["experts"], D, 2.0), rn(r["experts"], std=0.3)
+            if ml.get("shared"):
+                sd[q + "shared.sg"] = lin(1, D, 2.0)
+        if sdim:
+            sd[p + "side.gate"], sd[p + "side.proj"] = lin(sdim, D, 1.5), lin(D, sdim)
+            sd[p + "side.norm"] = rn(D, std=0.5)
+    return {k: v.bfloat16().float() for k, v in sd.items()}
+
+
+def router_margin(cfg, sd, tokens):
+    """Smallest gap, over all positions and routed layers, between the choice scores that decide the chosen set: the
+    last chosen and the first rejected expert, and the last kept and the first dropped group."""
+    W = {k: t64(v) for k, v in sd.items()}
+    eps = float(cfg["norm"]["eps"])
+    tok = torch.as_tensor(tokens, dtype=torch.long)
+    sdim = int((cfg.get("token_side") or {}).get("dim") or 0)
+    x = W["embed"][tok]
+    gap = math.inf
+    for i, l in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        h = token_shift(centred_norm(x, W[p + "norm1"], eps), W[p + "shift"])
+        x = x + (gla_mixer(h, W, p + "mix.", l["mixer"], eps) if l["type"] == "gla" else
+                 parallel_mixer(h, W, p + "mix.", l["mixer"], eps))
+        ml = l.get("mlp")
+        if ml is not None:
+            h = centred_norm(x, W[p + "norm2"], eps)
+            r = ml["router"]
+            E, top = r["experts"], r["top"]
+            c = torch.sigmoid(h @ W[p + "mlp.router"].T) + W[p + "mlp.correction"]
+            gr = r.get("groups") or {}
+            n, keep = int(gr.get("count") or 1), int(gr.get("keep") or 1)
+            if n > 1 and keep < n:
+                per = c.view(-1, n, E // n)
+                gs = per.topk(min(2, E // n), -1).values.sum(-1).sort(-1, descending=True).values
+                gap = min(gap, float((gs[:, keep - 1] - gs[:, keep]).min()))
+                ok = torch.zeros_like(gs, dtype=torch.bool).scatter_(
+                    1, per.topk(min(2, E // n), -1).values.sum(-1).topk(keep, -1).indices, True)
+                c = torch.where(ok[:, :, None].expand_as(per).reshape(-1, E), c, torch.full_like(c, -math.inf))
+            if top < E:
+                cs = c.sort(-1, descending=True).values
+                d = cs[:, top - 1] - cs[:, top]
+                gap = min(gap, float(d[torch.isfinite(d)].min()) if torch.isfinite(d).any() else math.inf)
+            x = x + moe(h, W, p + "mlp.", ml)
+        if sdim:
+            x = token_side(x, tok, W, i, sdim, eps)
+    return gap
