@@ -302,7 +302,7 @@ def test_prefill_decode_portions(device, dtype):
     assert len(got_res) == len(res)
     for i, (gr, wr) in enumerate(zip(got_res, res)):
         e = (gr.cpu().double() - wr).norm() / wr.norm()
-        assert e < (1e-5 if dtype == torch.float32 else 3e-2), (i, float(e))
+        assert e < (1e-5 if dtype == torch.float32 else 6e-2), (i, float(e))
 
 
 @pytest.mark.parametrize("device,dtype", TARGETS)
