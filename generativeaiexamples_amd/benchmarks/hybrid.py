@@ -1,4 +1,6 @@
 """Prefill and decode throughput of the hybrid decoders at layer sizes of real models (random weights), side by side:
+Vipolix (gated linear attention layers and layers of chunk-local attention beside a generalised delta rule, token shift,
+group-routed clamped experts plus a gated shared expert on every layer, a per-layer token input; fp32 residual / state),
 Lituvik (latent attention over a one-row-per-token cache, constant-decay linear attention, selective state-space scan,
 tanh norms, routed experts on the attention layers; fp32 residual / state), Ronavik (sigmoid attention beside a gated linear recurrence, state-space scan layers, sigmoid-routed experts, fp32
 post-norm residual / state), Pinavik (windowed attention + WKV + channel-decay delta rule, fp32 residual / state) and
@@ -26,10 +28,10 @@ SIZES = {  # name: (width, layers, ff, heads, head_dim)
 
 def add_args(ap):
     ap.add_argument("--hybrid", action="store_true",
-                    help="prefill / decode throughput of Lituvik, Ronavik, Pinavik and Qwen3-Next at equal layer sizes "
+                    help="prefill / decode throughput of Vipolix, Lituvik, Ronavik, Pinavik and Qwen3-Next at equal layer sizes "
                          "(one GPU)")
     ap.add_argument("--hybrid-sizes", default="1k,2k", help="comma list of " + ",".join(SIZES))
-    ap.add_argument("--hybrid-models", default="lituvik,ronavik,pinavik,qwen3-next")
+    ap.add_argument("--hybrid-models", default="vipolix,lituvik,ronavik,pinavik,qwen3-next")
     ap.add_argument("--hybrid-prefill", default="2048,8192", help="prompt lengths of the prefill measurement")
     ap.add_argument("--hybrid-decode", default="1,16,64", help="batch sizes of the decode measurement")
     ap.add_argument("--hybrid-context", type=int, default=1024)
@@ -38,6 +40,11 @@ def add_args(ap):
 
 def build(model: str, size: str, window: int, device):
     W, L, F, H, hd = SIZES[size]
+    if model == "vipolix":
+        from ..models.vipolix import VipolixConfig, VipolixModel
+
+        cfg = VipolixConfig.sized(W, L, F, H, hd, chunk=window, experts=8, top=2)
+        return VipolixModel(cfg, device=device).random_init(0)
     if model == "lituvik":
         from ..models.lituvik import LituvikConfig, LituvikModel
 

@@ -263,7 +263,7 @@ void unit_key_removal(const Tensor& k, const Tensor& a, const optional<Tensor>& 
 
 void dplr_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& decay, const optional<Tensor>& av,
                const optional<Tensor>& bv, Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& out,
-               double q_scale) {
+               double q_scale, const optional<Tensor>& ws) {
   const int dt = act_dt(q, "q");
   same_dt(k, dt, "k");
   same_dt(v, dt, "v");
@@ -274,9 +274,21 @@ void dplr_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& 
               "dplr_scan: q / k / decay [T, H * DK], v [T, H * DV], out [T, H, DV]");
   TORCH_CHECK(av.has_value() == bv.has_value(), "dplr_scan: the two removal vectors come together");
   if (av) TORCH_CHECK(av->numel() == decay.numel() && bv->numel() == decay.numel(), "dplr_scan: av / bv [T, H * DK]");
+  float* wsp = nullptr;
+  if (ws) {  // scratch of the chunk-parallel form
+    TORCH_CHECK(ws->is_cuda() && ws->scalar_type() == at::kFloat && ws->is_contiguous() &&
+                    (size_t)ws->numel() >= gai_dplr_scan_ws_floats(T, S, H, DK, DV, av ? 1 : 0),
+                "dplr_scan: chunk scratch too small");
+    wsp = ws->data_ptr<float>();
+  }
   gai_dplr_scan(q.data_ptr(), row_stride(q, "q"), k.data_ptr(), row_stride(k, "k"), v.data_ptr(), row_stride(v, "v"),
                 f32(decay, "decay"), av ? f32(*av, "av") : nullptr, bv ? f32(*bv, "bv") : nullptr, f32w(state, "state"),
-                i32(cu, "cu"), i32(slots, "slots"), S, T, f32w(out, "out"), H, DK, DV, (float)q_scale, dt, cur_stream());
+                i32(cu, "cu"), i32(slots, "slots"), S, T, f32w(out, "out"), H, DK, DV, (float)q_scale, dt, cur_stream(),
+                wsp);
+}
+
+int64_t dplr_scan_ws_floats(int64_t T, int64_t S, int64_t H, int64_t DK, int64_t DV, bool rank1) {
+  return (int64_t)gai_dplr_scan_ws_floats((int)T, (int)S, (int)H, (int)DK, (int)DV, rank1 ? 1 : 0);
 }
 
 void token_shift_mix(const Tensor& h, const Tensor& mu, const Tensor& shift_state, const Tensor& cu, const Tensor& slots,
@@ -561,6 +573,7 @@ void gai_bind_seq_ops(pybind11::module_& m) {
   m.def("decay_gate", &decay_gate);
   m.def("unit_key_removal", &unit_key_removal);
   m.def("dplr_scan", &dplr_scan);
+  m.def("dplr_scan_ws_floats", &dplr_scan_ws_floats);
   m.def("sigmoid_attention_splits", [](int64_t T, int64_t S, int64_t H) { return (int64_t)gai_sigmoid_attention_splits(T, S, H); });
   m.def("token_shift_mix", &token_shift_mix);
   m.def("state_tail_write", &state_tail_write);

@@ -263,7 +263,9 @@ void gai_unit_key_removal(const void* k, int ldk, const void* a, int lda, const 
 // S <- diag(decay) S - av (bv^T S) + k v^T (av = nullptr: no removal), o = q_scale S^T q
 void gai_dplr_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* decay,
                    const float* av, const float* bv, float* state, const int* cu, const int* slots, int S, int T,
-                   float* out, int H, int DK, int DV, float q_scale, int dt, hipStream_t st);
+                   float* out, int H, int DK, int DV, float q_scale, int dt, hipStream_t st, float* ws = nullptr);
+// fp32 elements of the scratch of the chunk-parallel form of such a step (0: the step runs unchunked)
+size_t gai_dplr_scan_ws_floats(int T, int S, int H, int DK, int DV, int rank1);
 void gai_token_shift_mix(const void* h, const float* mu, int NM, const float* shift_state, const int* cu,
                          const int* slots, int S, void* out, int T, int D, int dt, hipStream_t st);
 void gai_state_tail_write(const void* x, int ldx, float* state, const int* cu, const int* slots, int S, int C, int NR,

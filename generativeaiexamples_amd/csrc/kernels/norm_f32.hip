@@ -57,6 +57,50 @@ __global__ __launch_bounds__(256) void add_rmsnorm_f32_kernel(float* __restrict_
   for (int i = lane; i < D; i += 64) o[i] = (TA)(r[i] * inv * w[i]);
 }
 
+// Few rows (decode steps): one workgroup per row instead of one wave, the summed values kept in registers between the
+// passes (rows up to 256 * kAddWideRegs wide; wider rows re-read them).
+constexpr int kAddWideRegs = 16;
+
+template <typename TD, typename TA>
+__global__ __launch_bounds__(256) void add_rmsnorm_f32_wide_kernel(float* __restrict__ res, const TD* __restrict__ delta,
+                                                                   int ldd, float mult, const float* __restrict__ w,
+                                                                   TA* __restrict__ out, int D, float eps) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  float* r = res + (size_t)row * D;
+  const TD* d = delta ? delta + (size_t)row * ldd : nullptr;
+  float v[kAddWideRegs];
+  float s = 0.f;
+#pragma unroll
+  for (int q = 0; q < kAddWideRegs; ++q) {
+    const int i = tid + 256 * q;
+    v[q] = 0.f;
+    if (i < D) {
+      v[q] = d ? r[i] + mult * (float)d[i] : r[i];
+      if (d) r[i] = v[q];
+      s += v[q] * v[q];
+    }
+  }
+  for (int i = tid + 256 * kAddWideRegs; i < D; i += 256) {
+    const float x = d ? r[i] + mult * (float)d[i] : r[i];
+    if (d) r[i] = x;
+    s += x * x;
+  }
+  if (!out) return;
+  TA* o = out + (size_t)row * D;
+  float inv = 1.0f;
+  if (w) {
+    s = block_sum(s, scratch);
+    inv = 1.0f / sqrtf(s / D + eps);
+  }
+#pragma unroll
+  for (int q = 0; q < kAddWideRegs; ++q) {
+    const int i = tid + 256 * q;
+    if (i < D) o[i] = (TA)(w ? v[q] * inv * w[i] : v[q]);
+  }
+  for (int i = tid + 256 * kAddWideRegs; i < D; i += 256) o[i] = (TA)(w ? r[i] * inv * w[i] : r[i]);
+}
+
 template <typename TA>
 __global__ __launch_bounds__(256) void poly_norm_kernel(const TA* __restrict__ z, TA* __restrict__ y,
                                                         const float* __restrict__ coef, int F, float eps) {
@@ -399,12 +443,16 @@ void gai_add_rmsnorm_f32(float* res, const void* delta, int ldd, float mult, con
                          float eps, int dt_delta, int dt_out, hipStream_t st) {
   if (T == 0) return;
   const int grid = (T + 3) / 4;
-#define GAI_ARN(TD, TA) \
-  add_rmsnorm_f32_kernel<TD, TA><<<grid, 256, 0, st>>>(res, (const TD*)delta, ldd, mult, w, (TA*)out, T, D, eps)
-  if (dt_delta && dt_out) GAI_ARN(float, float);
-  else if (dt_delta) GAI_ARN(float, bf16);
-  else if (dt_out) GAI_ARN(bf16, float);
-  else GAI_ARN(bf16, bf16);
+  const bool wide = T <= 512 && D >= 512;  // few rows: a workgroup per row
+#define GAI_ARN(TD, TA)                                                                                              \
+  if (wide)                                                                                                          \
+    add_rmsnorm_f32_wide_kernel<TD, TA><<<T, 256, 0, st>>>(res, (const TD*)delta, ldd, mult, w, (TA*)out, D, eps);   \
+  else                                                                                                               \
+    add_rmsnorm_f32_kernel<TD, TA><<<grid, 256, 0, st>>>(res, (const TD*)delta, ldd, mult, w, (TA*)out, T, D, eps)
+  if (dt_delta && dt_out) { GAI_ARN(float, float); }
+  else if (dt_delta) { GAI_ARN(float, bf16); }
+  else if (dt_out) { GAI_ARN(bf16, float); }
+  else { GAI_ARN(bf16, bf16); }
 #undef GAI_ARN
   GAI_LAUNCH_CHECK();
 }

@@ -638,19 +638,56 @@ __global__ __launch_bounds__(1024) void dplr_scan_kernel(const TA* __restrict__ 
     if (i < nrow) Sg[(size_t)i * DV] = col[i];
 }
 
-template <typename TA, int R, int RGS, bool RANK1>
+// MODE 0: whole portions, state from / to the pool. A long portion of few sequences leaves most SIMDs without a wave, and
+// the recurrence is linear in S (S_t = A_t S_(t-1) + k_t v_t^T with A_t = diag(w_t) - av_t bv_t^T), so such a step is cut
+// into chunks of kDplrChunk tokens that run side by side:
+//   MODE 1: a chunk from a zero state, no outputs: its final state Q and its transition - without removal the product
+//           of its decays per key channel (P), with removal the DK x DK matrix M = A_n ... A_1, obtained by running the
+//           homogeneous recurrence on the columns of the identity (DK more columns of the same kernel, v = 0);
+//   carry:  per sequence S <- diag(P) S + Q or S <- M S + Q over its chunks, leaving every chunk's entry state in Q's
+//           place (and the pool's final state);
+//   MODE 2: the chunk again from its entry state, outputs written.
+// Only the association of the fp32 products differs from the serial order.
+constexpr int kDplrChunk = 256;
+
+__device__ __forceinline__ bool dplr_chunk_of(const int* __restrict__ cu, int S, int idx, int& s, int& t0, int& t1) {
+  int seen = 0;
+  for (s = 0; s < S; ++s) {
+    const int len = cu[s + 1] - cu[s], nc = (len + kDplrChunk - 1) / kDplrChunk;
+    if (idx < seen + nc) {
+      t0 = cu[s] + (idx - seen) * kDplrChunk;
+      t1 = min(t0 + kDplrChunk, cu[s + 1]);
+      return true;
+    }
+    seen += nc;
+  }
+  return false;
+}
+
+template <typename TA, int R, int RGS, bool RANK1, int MODE>
 __global__ __launch_bounds__(64) void dplr_scan_cols_kernel(const TA* __restrict__ q, int ldq, const TA* __restrict__ k,
                                                             int ldk, const TA* __restrict__ v, int ldv,
                                                             const float* __restrict__ decay, const float* __restrict__ av,
                                                             const float* __restrict__ bv, float* __restrict__ state,
                                                             const int* __restrict__ cu, const int* __restrict__ slots,
                                                             float* __restrict__ out, int H, int DK, int DV,
-                                                            float q_scale) {
+                                                            float q_scale, int S, float* __restrict__ Qbuf,
+                                                            float* __restrict__ Tbuf) {
   constexpr int COLS = 64 / RGS, NP = kTB * RGS * R / 64, LD = RGS * R + RGS, NA = RANK1 ? 5 : 3;
   extern __shared__ float lds[];
-  const int h = blockIdx.x, s = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
+  const int h = blockIdx.x, cb = blockIdx.z, lane = threadIdx.x;
+  int s = blockIdx.y, t0, t1;
+  if (MODE == 0) {
+    t0 = cu[s];
+    t1 = cu[s + 1];
+  } else if (!dplr_chunk_of(cu, S, blockIdx.y, s, t0, t1)) {
+    return;
+  }
   const int jj = lane / RGS, rg = lane % RGS, j = cb * COLS + jj;
-  const bool on = j < DV;
+  // MODE 1 with removal: columns DV .. DV + DK - 1 are the columns of the chunk's transition matrix
+  const bool is_m = MODE == 1 && RANK1 && j >= DV;
+  const int jm = j - DV;
+  const bool on = j < DV || (is_m && jm < DK);
   const int row0 = rg * R, nrow = max(0, min(R, DK - row0));
   float* qs = lds;
   float* ks = qs + kTB * LD;
@@ -658,13 +695,21 @@ __global__ __launch_bounds__(64) void dplr_scan_cols_kernel(const TA* __restrict
   float* as = ws + kTB * LD;     // RANK1 only
   float* bs = as + kTB * LD;
   float* vs = lds + NA * kTB * LD;  // [kTB][COLS]
-  const int t0 = cu[s], t1 = cu[s + 1];
   if (t1 <= t0) return;
   for (int x = lane; x < NA * kTB * LD; x += 64) lds[x] = 0.f;
-  float* Sg = state + (((size_t)slots[s] * H + h) * DK + row0) * DV + j;
-  float col[R];
+  // MODE 0: the pool's slot; MODE 1 / 2: the chunk's own [H, DK, DV] image in Qbuf (MODE 2 reads its entry state
+  // there), the transition matrix columns in Tbuf [chunk, H, DK, DK]
+  const int lds_s = is_m ? DK : DV;
+  float* Sg = MODE == 0 ? state + (((size_t)slots[s] * H + h) * DK + row0) * DV + j
+              : is_m    ? Tbuf + (((size_t)blockIdx.y * H + h) * DK + row0) * DK + jm
+                        : Qbuf + (((size_t)blockIdx.y * H + h) * DK + row0) * DV + j;
+  float col[R], pprod[(MODE == 1 && !RANK1) ? R : 1];
 #pragma unroll
-  for (int i = 0; i < R; ++i) col[i] = (on && i < nrow) ? Sg[(size_t)i * DV] : 0.f;
+  for (int i = 0; i < R; ++i) {
+    if (MODE == 1) col[i] = (is_m && row0 + i == jm) ? 1.f : 0.f;
+    else col[i] = (on && i < nrow) ? Sg[(size_t)i * lds_s] : 0.f;
+    if (MODE == 1 && !RANK1) pprod[i] = 1.f;
+  }
   constexpr int NPART = 64 / kTB;
   static_assert(NP * NPART >= RGS * R, "staging covers a full row");
   const int stt = lane / NPART, spart = lane % NPART;
@@ -738,18 +783,98 @@ __global__ __launch_bounds__(64) void dplr_scan_cols_kernel(const TA* __restrict
         }
         col[i] = c0;
         col[i + 1] = c1;
-        o0 = fmaf(c0, qs[a + i], o0);
-        o1 = fmaf(c1, qs[a + i + 1], o1);
+        if (MODE == 1 && !RANK1) {
+          pprod[i] *= ws[a + i];
+          pprod[i + 1] *= ws[a + i + 1];
+        }
+        if (MODE != 1) {
+          o0 = fmaf(c0, qs[a + i], o0);
+          o1 = fmaf(c1, qs[a + i + 1], o1);
+        }
       }
-      const float oo = rowgroup_sum<RGS>(o0 + o1);
-      if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * DV + j] = oo * q_scale;
+      if (MODE != 1) {
+        const float oo = rowgroup_sum<RGS>(o0 + o1);
+        if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * DV + j] = oo * q_scale;
+      }
     }
   }
-  if (on) {
+  if (on && MODE != 2) {
 #pragma unroll
     for (int i = 0; i < R; ++i)
-      if (i < nrow) Sg[(size_t)i * DV] = col[i];
+      if (i < nrow) Sg[(size_t)i * lds_s] = col[i];
   }
+  if (MODE == 1 && !RANK1 && cb == 0 && jj == 0) {  // the chunk's decay product per key channel
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (i < nrow) Tbuf[((size_t)blockIdx.y * H + h) * DK + row0 + i] = pprod[i];
+  }
+}
+
+// S <- diag(P) S + Q over the chunks of a sequence; Q[chunk] is replaced by the chunk's entry state
+__global__ __launch_bounds__(256) void dplr_chunk_carry_diag_kernel(const float* __restrict__ Pbuf, float* __restrict__ Qbuf,
+                                                                    float* __restrict__ state, const int* __restrict__ cu,
+                                                                    const int* __restrict__ slots, int H, int DK, int DV) {
+  const int e = blockIdx.x * 256 + threadIdx.x, h = blockIdx.y, s = blockIdx.z, ND = DK * DV;
+  if (e >= ND) return;
+  const int len = cu[s + 1] - cu[s];
+  if (len <= 0) return;
+  int first = 0;
+  for (int x = 0; x < s; ++x) first += (cu[x + 1] - cu[x] + kDplrChunk - 1) / kDplrChunk;
+  const int nc = (len + kDplrChunk - 1) / kDplrChunk, row = e / DV;
+  float* sp = state + ((size_t)slots[s] * H + h) * ND + e;
+  float Sv = *sp;
+  for (int n = 0; n < nc; ++n) {
+    float* qp = Qbuf + ((size_t)(first + n) * H + h) * ND + e;
+    const float qv = *qp;
+    *qp = Sv;
+    Sv = fmaf(Pbuf[((size_t)(first + n) * H + h) * DK + row], Sv, qv);
+  }
+  *sp = Sv;
+}
+
+// S <- M S + Q over the chunks of a sequence (M: the chunk's DK x DK transition); one workgroup per (block of kCarryCols
+// state columns, head, sequence), thread r owns row r of the block, the block's current S sits in LDS
+constexpr int kCarryCols = 16;
+
+__global__ __launch_bounds__(256) void dplr_chunk_carry_full_kernel(const float* __restrict__ Mbuf, float* __restrict__ Qbuf,
+                                                                    float* __restrict__ state, const int* __restrict__ cu,
+                                                                    const int* __restrict__ slots, int H, int DK, int DV) {
+  extern __shared__ float Sc[];  // [DK][kCarryCols]
+  const int c0 = blockIdx.x * kCarryCols, h = blockIdx.y, s = blockIdx.z, r = threadIdx.x;
+  const int len = cu[s + 1] - cu[s];
+  if (len <= 0) return;
+  int first = 0;
+  for (int x = 0; x < s; ++x) first += (cu[x + 1] - cu[x] + kDplrChunk - 1) / kDplrChunk;
+  const int nc = (len + kDplrChunk - 1) / kDplrChunk, ncol = min(kCarryCols, DV - c0);
+  float* sp = state + (((size_t)slots[s] * H + h) * DK + r) * DV + c0;
+  if (r < DK)
+    for (int c = 0; c < kCarryCols; ++c) Sc[r * kCarryCols + c] = c < ncol ? sp[c] : 0.f;
+  __syncthreads();
+  for (int n = 0; n < nc; ++n) {
+    float acc[kCarryCols];
+    if (r < DK) {
+      float* qp = Qbuf + (((size_t)(first + n) * H + h) * DK + r) * DV + c0;
+#pragma unroll
+      for (int c = 0; c < kCarryCols; ++c) {
+        acc[c] = c < ncol ? qp[c] : 0.f;
+        if (c < ncol) qp[c] = Sc[r * kCarryCols + c];
+      }
+      const float* mr = Mbuf + (((size_t)(first + n) * H + h) * DK + r) * DK;
+      for (int kk = 0; kk < DK; ++kk) {
+        const float m = mr[kk];
+#pragma unroll
+        for (int c = 0; c < kCarryCols; ++c) acc[c] = fmaf(m, Sc[kk * kCarryCols + c], acc[c]);
+      }
+    }
+    __syncthreads();
+    if (r < DK) {
+#pragma unroll
+      for (int c = 0; c < kCarryCols; ++c) Sc[r * kCarryCols + c] = acc[c];
+    }
+    __syncthreads();
+  }
+  if (r < DK)
+    for (int c = 0; c < ncol; ++c) sp[c] = Sc[r * kCarryCols + c];
 }
 
 // ---- real-gated linear recurrent unit -----------------------------------------------------------------------------
@@ -1616,21 +1741,50 @@ void gai_unit_key_removal(const void* k, int ldk, const void* a, int lda, const 
   GAI_LAUNCH_CHECK();
 }
 
+// fp32 elements of the scratch that the chunked scan of such a step needs (0: the step runs unchunked)
+size_t gai_dplr_scan_ws_floats(int T, int S, int H, int DK, int DV, int rank1) {
+  const int RGS = DK <= 64 ? 8 : 16;
+  const long waves = (long)H * S * ((DV + 64 / RGS - 1) / (64 / RGS));
+  if (T <= S || T < 2 * kDplrChunk || waves >= 4096) return 0;  // single tokens, short portions, or SIMDs already full
+  const size_t NC = (size_t)T / kDplrChunk + S;
+  return NC * H * ((size_t)DK * DV + (rank1 ? (size_t)DK * DK : (size_t)DK));
+}
+
 void gai_dplr_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* decay,
                    const float* av, const float* bv, float* state, const int* cu, const int* slots, int S, int T,
-                   float* out, int H, int DK, int DV, float q_scale, int dt, hipStream_t st) {
+                   float* out, int H, int DK, int DV, float q_scale, int dt, hipStream_t st, float* ws) {
   if (S == 0 || T == 0) return;
   if (DK > kMaxDK) gai_launch_error(__FILE__, __LINE__, "dplr_scan: key head size above 256");
   if ((av == nullptr) != (bv == nullptr)) gai_launch_error(__FILE__, __LINE__, "dplr_scan: the two removal vectors come together");
   const bool r1 = av != nullptr;
   if (T > S) {  // some sequence brings more than one row: the column-sliced scan
+    const bool chunked = ws && gai_dplr_scan_ws_floats(T, S, H, DK, DV, r1) > 0;
+    const int NC = T / kDplrChunk + S;
+    float* Qbuf = ws;
+    float* Tbuf = ws ? ws + (size_t)NC * H * DK * DV : nullptr;
+#define GAI_DPLR_L(TA, R, RGS, R1, MODE, NY, NCOL)                                                                   \
+  do {                                                                                                               \
+    const dim3 grid(H, NY, ((NCOL) + 64 / RGS - 1) / (64 / RGS));                                                    \
+    const size_t lds = (size_t)((R1 ? 5 : 3) * kTB * (RGS * R + RGS) + kTB * (64 / RGS)) * sizeof(float);            \
+    dplr_scan_cols_kernel<TA, R, RGS, R1, MODE><<<grid, 64, lds, st>>>(                                              \
+        (const TA*)q, ldq, (const TA*)k, ldk, (const TA*)v, ldv, decay, av, bv, state, cu, slots, out, H, DK, DV,    \
+        q_scale, S, Qbuf, Tbuf);                                                                                     \
+  } while (0)
 #define GAI_DPLR_C(TA, R, RGS, R1)                                                                                   \
   do {                                                                                                               \
-    const dim3 grid(H, S, (DV + 64 / RGS - 1) / (64 / RGS));                                                         \
-    const size_t lds = (size_t)((R1 ? 5 : 3) * kTB * (RGS * R + RGS) + kTB * (64 / RGS)) * sizeof(float);            \
-    dplr_scan_cols_kernel<TA, R, RGS, R1><<<grid, 64, lds, st>>>((const TA*)q, ldq, (const TA*)k, ldk, (const TA*)v, \
-                                                                 ldv, decay, av, bv, state, cu, slots, out, H, DK,   \
-                                                                 DV, q_scale);                                       \
+    if (chunked) {                                                                                                   \
+      GAI_DPLR_L(TA, R, RGS, R1, 1, NC, R1 ? DV + DK : DV);                                                          \
+      if (R1)                                                                                                        \
+        dplr_chunk_carry_full_kernel<<<dim3((DV + kCarryCols - 1) / kCarryCols, H, S), 256,                          \
+                                       (size_t)DK * kCarryCols * sizeof(float), st>>>(Tbuf, Qbuf, state, cu, slots,  \
+                                                                                      H, DK, DV);                    \
+      else                                                                                                           \
+        dplr_chunk_carry_diag_kernel<<<dim3((DK * DV + 255) / 256, H, S), 256, 0, st>>>(Tbuf, Qbuf, state, cu,       \
+                                                                                       slots, H, DK, DV);            \
+      GAI_DPLR_L(TA, R, RGS, R1, 2, NC, DV);                                                                         \
+    } else {                                                                                                         \
+      GAI_DPLR_L(TA, R, RGS, R1, 0, S, DV);                                                                          \
+    }                                                                                                                \
   } while (0)
 #define GAI_DPLR_S(TA, R1)                                                                                           \
   do {                                                                                                               \
@@ -1641,6 +1795,7 @@ void gai_dplr_scan(const void* q, int ldq, const void* k, int ldk, const void* v
     else { if (r1) GAI_DPLR_S(bf16, true); else GAI_DPLR_S(bf16, false); }
 #undef GAI_DPLR_S
 #undef GAI_DPLR_C
+#undef GAI_DPLR_L
     GAI_LAUNCH_CHECK();
     return;
   }

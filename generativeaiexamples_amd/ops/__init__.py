@@ -1477,5 +1477,8 @@ def dplr_scan(q, k, v, decay, av, bv, state, cu, slots, q_scale: float = 1.0):
         return ref.dplr_scan(q, k, v, decay, av, bv, state, cu, slots, q_scale)
     H, DV = state.shape[1], state.shape[3]
     out = torch.empty(q.shape[0], H, DV, dtype=torch.float32, device=q.device)
-    native().dplr_scan(q, k, v, decay, av, bv, state, cu, slots, out, float(q_scale))
+    # long portions of few sequences run chunk-parallel through a scratch (chunk states and chunk transitions)
+    nws = native().dplr_scan_ws_floats(q.shape[0], slots.numel(), H, state.shape[2], DV, av is not None)
+    ws = torch.empty(nws, dtype=torch.float32, device=q.device) if nws else None
+    native().dplr_scan(q, k, v, decay, av, bv, state, cu, slots, out, float(q_scale), ws)
     return out

@@ -481,6 +481,60 @@ def test_matrix_core_kernels_in_model():
         assert close(got[n], want[n], torch.bfloat16), n
 
 
+@_GPU
+@pytest.mark.parametrize("removal", [False, True], ids=["decay-only", "with-removal"])
+@pytest.mark.parametrize("H,dk,dv", [(2, 16, 24), (1, 70, 9), (2, 130, 20), (3, 64, 64)])
+def test_chunk_parallel_scan_against_serial(H, dk, dv, removal):
+    """Long portions of few sequences run the scan chunk-parallel (chunk states, chunk transitions, a carry pass): same
+    outputs and final states as the serial recurrence in float64, from states that are not zero, with a sequence that
+    ends inside a chunk and a single token beside them."""
+    g = torch.Generator().manual_seed(3)
+    rn = lambda *s: torch.randn(*s, generator=g)  # noqa: E731
+    cu_l = [0, 700, 1300, 1301]
+    T = cu_l[-1]
+    n = 2 * H * dk + H * dv
+    qkv, st = rn(T, n) * 0.5, rn(5, H, dk, dv)
+    dec = 1.0 - 0.1 * torch.rand(T, H * dk, generator=g)
+    u = rn(T, H, dk)
+    u = (u / u.norm(dim=-1, keepdim=True)).reshape(T, H * dk)
+    a_ = u * torch.rand(T, H * dk, generator=g)
+    dev = torch.device("cuda")
+    cu, slots = torch.tensor(cu_l, dtype=torch.int32, device=dev), torch.tensor([3, 0, 4], dtype=torch.int32, device=dev)
+    s_dev, buf = st.clone().to(dev), qkv.to(dev)
+    assert ops.native().dplr_scan_ws_floats(T, 3, H, dk, dv, removal) > 0
+    got = ops.dplr_scan(buf[:, :H * dk], buf[:, H * dk:2 * H * dk], buf[:, 2 * H * dk:], dec.to(dev),
+                        a_.to(dev) if removal else None, u.to(dev) if removal else None, s_dev, cu, slots).cpu().double()
+    r3 = lambda t, d: t.double().reshape(T, H, d)  # noqa: E731
+    q3, k3, v3 = r3(qkv[:, :H * dk], dk), r3(qkv[:, H * dk:2 * H * dk], dk), r3(qkv[:, 2 * H * dk:], dv)
+    w3, a3, b3 = r3(dec, dk), r3(a_, dk), r3(u, dk)
+    for i, sl in enumerate([3, 0, 4]):
+        S = st[sl].double()
+        for t in range(cu_l[i], cu_l[i + 1]):
+            new = w3[t][:, :, None] * S + k3[t][:, :, None] * v3[t][:, None, :]
+            if removal:
+                new = new - a3[t][:, :, None] * torch.einsum("hk,hkv->hv", b3[t], S)[:, None, :]
+            S = new
+            want = torch.einsum("hkv,hk->hv", S, q3[t])
+            assert torch.allclose(got[t], want, atol=5e-4, rtol=5e-4), (t, float((got[t] - want).abs().max()))
+        assert torch.allclose(s_dev[sl].cpu().double(), S, atol=5e-4, rtol=5e-4)
+    assert torch.equal(s_dev[1].cpu(), st[1]) and torch.equal(s_dev[2].cpu(), st[2])
+
+
+@_GPU
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_long_prompt_against_oracle(dtype):
+    """A prompt long enough for the chunk-parallel scans (and several chunks of the attention mask), whole and cut in
+    two, against the oracle at every position."""
+    cfg = config_for(dtype, [O.moe_ff(O.gla(heads=2, dim=16, vdim=16)), O.no_ff(O.par(chunk=100, rheads=2, rdim=16))])
+    sd = O.random_checkpoint(cfg, 41)
+    toks = clear_tokens(640, cfg, sd, 42)
+    want = O.forward(cfg, sd, toks)
+    eng = make_engine(cfg, sd, "cuda", dtype, max_tokens=1024)
+    for name, sizes in (("whole", [640]), ("two", [530, 110])):
+        got = run_schedule(eng, {name: toks}, [[(name, c)] for c in sizes])[name]
+        assert close(got, want, dtype), name
+
+
 @pytest.mark.parametrize("device,dtype", TARGETS)
 @pytest.mark.parametrize("shape", ["wide-odd", "tiny", "no-side-no-shift"])
 def test_other_shapes(shape, device, dtype):
