@@ -5,7 +5,8 @@
 namespace gai {
 
 enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_BIAS_GELU = 2, EPI_RESIDUAL = 3, EPI_SWIGLU = 4, EPI_BIAS_RESIDUAL = 5,
-       EPI_BIAS_RELU = 6, EPI_BIAS_QUICKGELU = 7, EPI_RELU2 = 8 };
+       EPI_BIAS_RELU = 6, EPI_BIAS_QUICKGELU = 7, EPI_RELU2 = 8,
+       EPI_CLAMP_GLU = 9 /* [gate16 | up16] rows: min(g, p) sigmoid(1.702 min(g, p)) (clamp(u, +-p) + 1) */ };
 
 __device__ __forceinline__ float quick_gelu(float x) { return x / (1.0f + __expf(-1.702f * x)); }
 

@@ -137,9 +137,9 @@ void gai_ep_pack(const void* x, const int* ids, const int* offs, const int* a_pa
 void gai_ep_combine(const void* back, const int* ids, const int* pos, const int* offs, const float* w,
                     const void* residual, void* out, int T, int k, int D, int e_local, int C, hipStream_t st);
 // gemm_decode.hip: decode-sized grouped GEMM on the weight-streaming decode kernel (0 = shape not handled)
-// act: 0 none, 1 SwiGLU on the [gate16 | up16] interleave, 2 squared ReLU
+// act: 0 none, 1 SwiGLU on the [gate16 | up16] interleave, 2 squared ReLU, 3 clamped gated (limit actp, same interleave)
 int gai_moe_gemm_dec2(const void* A, const int* a_rows, const void* W, void* C, const int* offs, int E,
-                      int rows_total, int N, int K, int act, hipStream_t st);
+                      int rows_total, int N, int K, int act, hipStream_t st, float actp = 0.f);
 // sigmoid: scores sigmoid(logit) per expert instead of a softmax over the experts (weights = the chosen scores)
 void gai_moe_route(const float* logits, int T, int E, int k, int renorm, int* ids, float* w, hipStream_t st,
                    int sigmoid = 0, const float* bias = nullptr, float eps = 0.f);

@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_dec2_kernel(const bf16* __re
                                                                 void* C, const bf16* __restrict__ bias, const bf16* R,
                                                                 int M, int N, int K, int ldc, float* __restrict__ part,
                                                                 const int* __restrict__ moe_rows,
-                                                                const int* __restrict__ moe_offs) {
+                                                                const int* __restrict__ moe_offs, float epi_param) {
   constexpr int KQ = 8 / NT;
   int row0 = 0;
   if (moe_offs != nullptr) {  // wave-uniform: the whole workgroup leaves before any barrier when the expert is idle
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_dec2_kernel(const bf16* __re
       }
       dec_store8<true>(part, ((size_t)ks * M + m) * N + n, v);
     }
-  } else if (EPI == EPI_SWIGLU) {
+  } else if (EPI == EPI_SWIGLU || EPI == EPI_CLAMP_GLU) {
     // 16-column tiles (2j, 2j + 1) are (gate, up); output columns nb / 2 + 16 j + 8 h .. + 7
     constexpr int ITEMS = ROWS * NT;  // (m, j, h)
     for (int e = tid; e < ITEMS; e += kThreads) {
@@ -239,7 +239,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_dec2_kernel(const bf16* __re
           g += red[(q * ROWS + m) * RS + gc + x];
           up += red[(q * ROWS + m) * RS + gc + 16 + x];
         }
-        v[x] = silu(g) * up;
+        if (EPI == EPI_CLAMP_GLU) {
+          g = fminf(g, epi_param);
+          up = fminf(fmaxf(up, -epi_param), epi_param);
+          v[x] = g / (1.0f + expf(-1.702f * g)) * (up + 1.0f);
+        } else {
+          v[x] = silu(g) * up;
+        }
       }
       dec_store8<OUTF32>(C, (size_t)m * ldc + nb / 2 + 16 * j + 8 * h, v);
     }
@@ -273,7 +279,7 @@ constexpr int dec2_steps_multiple() { return DecCfg<MB, 8 / NT>::L; }
 template <int MB, int NT, int EPI, bool OUTF32, bool PART = false, bool PSW = false>
 void dec2_launch(const void* A, const void* W, void* C, const void* bias, const void* R, int M, int N, int K, int ldc,
                  hipStream_t st, int KS = 1, float* part = nullptr, const int* moe_rows = nullptr,
-                 const int* moe_offs = nullptr, int E = 1) {
+                 const int* moe_offs = nullptr, int E = 1, float epi_param = 0.f) {
   auto kern = gemm_dec2_kernel<MB, NT, EPI, OUTF32, PART, PSW>;
   constexpr int lds = 2 * kStage;
   static bool once = false;
@@ -283,7 +289,7 @@ void dec2_launch(const void* A, const void* W, void* C, const void* bias, const 
   }
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
   kern<<<dim3(blocks, KS, E), kThreads, lds, st>>>((const bf16*)A, (const bf16*)W, C, (const bf16*)bias,
-                                                   (const bf16*)R, M, N, K, ldc, part, moe_rows, moe_offs);
+                                                   (const bf16*)R, M, N, K, ldc, part, moe_rows, moe_offs, epi_param);
   GAI_LAUNCH_CHECK();
 }
 
@@ -473,8 +479,9 @@ int gai_gemm_dec2_partials(const void* A, const void* W, int M, int N, int K, fl
 // for a handful of live ones and keep one 32 KB stage in flight per CU. swiglu: W rows interleaved per 16
 // [gate16 | up16] (ops.interleave_gate_up), C = silu(gate) * up. Returns 0 when the shape does not fit.
 int gai_moe_gemm_dec2(const void* A, const int* a_rows, const void* W, void* C, const int* offs, int E,
-                      int rows_total, int N, int K, int act, hipStream_t st) {
-  const int swiglu = act == 1, relu2 = act == 2;  // act: 0 none, 1 SwiGLU, 2 squared ReLU
+                      int rows_total, int N, int K, int act, hipStream_t st, float actp) {
+  // act: 0 none, 1 SwiGLU, 2 squared ReLU, 3 clamped gated (limit actp; the row interleave of SwiGLU)
+  const int swiglu = act == 1 || act == 3, relu2 = act == 2, clampg = act == 3;
   if (rows_total < 1 || rows_total > 64 || N % 32) return 0;
   const int ldc = swiglu ? N / 2 : N;
   const int epi = swiglu ? EPI_SWIGLU : EPI_NONE;
@@ -485,9 +492,14 @@ int gai_moe_gemm_dec2(const void* A, const int* a_rows, const void* W, void* C, 
     auto go = [&](auto ntc) {                                                                                     \
       constexpr int NTV = decltype(ntc)::value;                                                                   \
       if (epi == EPI_SWIGLU) {                                                                                    \
-        if constexpr (NTV >= 2)                                                                                   \
-          dec2_launch<MBV, NTV, EPI_SWIGLU, false>(A, W, C, nullptr, nullptr, rows_total, N, K, ldc, st, 1,       \
-                                                   nullptr, a_rows, offs, E);                                     \
+        if constexpr (NTV >= 2) {                                                                                 \
+          if (clampg)                                                                                             \
+            dec2_launch<MBV, NTV, EPI_CLAMP_GLU, false>(A, W, C, nullptr, nullptr, rows_total, N, K, ldc, st, 1,  \
+                                                        nullptr, a_rows, offs, E, actp);                          \
+          else                                                                                                    \
+            dec2_launch<MBV, NTV, EPI_SWIGLU, false>(A, W, C, nullptr, nullptr, rows_total, N, K, ldc, st, 1,     \
+                                                     nullptr, a_rows, offs, E);                                   \
+        }                                                                                                         \
       } else if (relu2) {                                                                                         \
         dec2_launch<MBV, NTV, EPI_RELU2, false>(A, W, C, nullptr, nullptr, rows_total, N, K, ldc, st, 1, nullptr, \
                                                 a_rows, offs, E);                                                 \

@@ -613,8 +613,7 @@ void gai_moe_gemm(const void* A, const int* a_rows, const void* W, void* C, cons
     return;
   }
   // decode steps (<= 64 expert rows in all): every expert's weights streamed once by the decode kernel
-  // (the clamped gated epilogue lives in the tiled kernels only)
-  if (act != 3 && gai_moe_gemm_dec2(A, a_rows, W, C, offs, E, rows_total, N, K, act, st)) return;
+  if (gai_moe_gemm_dec2(A, a_rows, W, C, offs, E, rows_total, N, K, act, st, actp)) return;
   const dim3 grid((rows_total + MBM - 1) / MBM + E, (N + MBN - 1) / MBN);
   const int lds = 4 * kMTile;
   static bool once = false;
