@@ -17,8 +17,8 @@
 // moe_route (choice bias): the experts are chosen by softmax score + bias_e while the weights stay the plain scores,
 //              renormalised over the chosen ones (+ eps in the sum); libm expf, all fp32.
 // moe_combine (identity experts): a chosen id >= n_real has no weights - its output is the token's own input row.
-// moe_route (grouped sigmoid): choice on sigmoid score + bias among the experts of the best groups (a group scores the
-//              sum of its two largest choice scores); weights = the chosen plain scores renormalised (+ eps), scaled.
+// moe_route (grouped sigmoid): choice on sigmoid score + bias confined to the best contiguous expert groups (ranked by their
+//              top-2 choice scores added up); weights = the chosen plain scores renormalised (+ eps), scaled.
 // moe_gemm (clamped gated): g = min(gate, p), u = clamp(up, +-p), g sigmoid(1.702 g) (u + 1) on [gate16 | up16] rows.
 // moe_combine (residual gate): the residual row (a shared expert's output) times sigmoid of a per-token logit.
 // moe_scale_rows: expert-sorted copies of the token rows, each times its routing weight (experts whose routing weight
@@ -92,8 +92,8 @@ __device__ __forceinline__ float glu_pair(float g, float u, float p) {
 }
 
 // Sigmoid scores with a choice correction and group-limited top-k, one lane per token: choice score c_e = sigmoid(x_e) +
-// bias_e; the experts form NG equal groups of neighbours, a group scores the sum of its two largest choice scores, only
-// experts of the KEEP best groups can be chosen (NG <= 64: the kept groups are a bit mask); the weights are the chosen
+// bias_e; the expert list is cut into NG contiguous groups of equal size, each ranked by its top-2 choice scores added up, and
+// the choice is confined to the KEEP best groups (NG <= 64: the kept groups are a bit mask); the weights are the chosen
 // plain scores over their sum (+ eps), times scale. All fp32, libm expf.
 __global__ void moe_route_grouped_kernel(const float* __restrict__ logits, int T, int E, int k, int* __restrict__ ids,
                                          float* __restrict__ w, const float* __restrict__ bias, float eps, int NG,

@@ -24,8 +24,8 @@
 //   decay_gate        token-parallel fp32 gates of a recurrence from their logits: sigmoid(x), sigmoid(x)^(1 / p) (through
 //                     its logarithm -softplus(-x) / p) or exp(-p sigmoid(x))
 //   unit_key_removal  per head the unit key u = k / sqrt(sum k^2 + eps) and the removal vector sigmoid(a + bias) * u
-//   dplr_scan         diagonal decay plus a rank-one removal: S <- diag(w_t) S - av_t (bv_t^T S) + k_t v_t^T (both terms
-//                     read the old state), o_t = scale * S^T q_t; without av / bv it is gated linear attention
+//   dplr_scan         diagonal decay plus a rank-one removal: S <- diag(w_t) S - av_t (bv_t^T S) + k_t v_t^T (decay and removal
+//                     both act on S_(t-1)), o_t = scale * S^T q_t; without av / bv it is gated linear attention
 //
 // A batch is S sequences of rows [cu[s], cu[s+1]) with pool slot slots[s] (device vectors: graph-capturable); a decoded
 // token is a sequence of one row, a prompt portion a longer one. The scans keep the state in VGPRs for the whole

@@ -4,8 +4,8 @@ and a per-layer token input.
 
 Architecture (every size and constant comes from ``config.json``; the layer list may hold the mixers in any order):
   * token embedding; the output head is its own matrix;
-  * a layer is pre-norm: ``x += mixer(shift(N1(x)))`` then ``x += ff(N2(x))``; the norm is an RMS norm whose weight is
-    stored around zero (``* (1 + w)``); a layer may have no feed-forward;
+  * a layer is pre-norm: ``x += mixer(shift(N1(x)))`` then ``x += ff(N2(x))``; the norm is an RMS norm with a
+    zero-centred weight (``* (1 + w)``); a layer may have no feed-forward;
   * token shift: the mixer reads ``h_t + (h_(t-1) - h_t) * mu`` (zeros before the first token);
   * per-layer token input, after the feed-forward: the layer's slice e of a second embedding of the token,
     ``y = W_proj (gelu_tanh(W_gate x) * e)``, ``x += rmsnorm(y) * w``;
@@ -15,7 +15,7 @@ Architecture (every size and constant comes from ``config.json``; the layer list
   * mixer ``parallel``: two branches on the same input, added with fixed scales. Left: GQA with biases and a short
     causal convolution on q, k and v, a rotation of the first ``rot.dims`` channels of each head in interleaved pairs,
     a temperature per head, keys visible only inside the query's own chunk of ``mask.size`` positions, and a softmax
-    with one added to the denominator. Right: the generalised delta rule ``S <- diag(w) S - (a * u)(u^T S) + k v^T``
+    whose denominator carries an extra 1 (a value-less sink of score 0). Right: the generalised delta rule ``S <- diag(w) S - (a * u)(u^T S) + k v^T``
     with the unit key u, decay ``w = exp(-e^(-1/2) sigmoid(.))`` and removal rate ``a = sigmoid(.)`` per key channel;
     per-head unit RMS, a weight over all heads, a sigmoid gate;
   * feed-forward: a mixture of experts with a sigmoid router - the choice made on ``score + correction`` among the

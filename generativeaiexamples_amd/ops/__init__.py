@@ -832,8 +832,8 @@ def moe_route(logits: torch.Tensor, k: int, renorm: bool = True, score: str = "s
     renormalised over the chosen experts) or "sigmoid" (each expert scored alone; weights are the chosen scores).
     bias (fp32 [E], softmax scoring): the experts are chosen by score + bias while the weights stay the plain scores;
     eps is added to the sum that renormalises them. Sigmoid scoring with bias, groups or scale: the choice is made on
-    sigmoid score + bias; groups = (count, keep) cuts the experts into `count` equal groups of neighbours, scores a
-    group by the sum of its two largest choice scores and lets only experts of the `keep` best groups be chosen; the
+    sigmoid score + bias; groups = (count, keep) cuts the expert list into `count` contiguous parts of equal size, ranks
+    each by its two best choice scores added up and confines the choice to the `keep` best parts; the
     weights are the chosen plain scores over their sum (+ eps), times scale."""
     if score not in ("softmax", "sigmoid"):
         raise ValueError(f"moe_route: unknown score function {score!r}")
@@ -1470,7 +1470,7 @@ def unit_key_removal(k, a, a_bias, H: int, DK: int, eps: float):
 def dplr_scan(q, k, v, decay, av, bv, state, cu, slots, q_scale: float = 1.0):
     """Linear recurrence with a diagonal decay plus a rank-one removal, per head:
     S_t = diag(decay_t) S_(t-1) - av_t (bv_t^T S_(t-1)) + k_t v_t^T,  o_t = q_scale * S_t^T q_t
-    (both terms read the old state; av / bv None: gated linear attention). q / k [T, H * DK] and v [T, H * DV] in the
+    (decay and removal both act on S_(t-1); av / bv None: gated linear attention). q / k [T, H * DK] and v [T, H * DV] in the
     activation dtype (column slices of a projection), decay / av / bv fp32 [T, H * DK]; state [slots, H, DK, DV] fp32 in
     place -> fp32 [T, H, DV]."""
     if not q.is_cuda:

@@ -1007,8 +1007,8 @@ def dplr_scan(q, k, v, decay, av, bv, state, cu, slots, q_scale):
 
 
 def moe_route_grouped(logits, k, bias, eps, groups, keep, scale, group_top=2):
-    """Sigmoid scores s; choice scores s + bias; the experts form `groups` equal groups of neighbours, a group scores
-    the sum of its group_top largest choice scores and only experts of the `keep` best groups can be chosen; weights
+    """Sigmoid scores s; choice scores s + bias; the expert list is cut into `groups` contiguous parts of
+    equal size, each ranked by its group_top best choice scores added up, and the choice is confined to the `keep` best parts; weights
     s / (sum of the chosen s + eps) * scale."""
     s = torch.sigmoid(logits.float())
     c = s + bias.float() if bias is not None else s.clone()

@@ -17,7 +17,7 @@ Prefill steps (``exact_counts=True``) exchange the per-destination pair counts f
 peer-memory all-to-all), and the slab exchange then moves only each segment's valid rows over xGMI
 (CustomAllReduce.all_to_all send_rows / recv_rows); rows past a peer's count are marked padding on the receiver.
 So prefill moves the exact bytes of the old count-then-variable-split exchange without its host round trip
-(round 4 copied the bincount of the destinations to the host: one device sync per MoE layer). Over
+(an earlier form copied the bincount of the destinations to the host: one device sync per MoE layer). Over
 RCCL (slabs beyond the peer buffers, or no peer exchange) the equal-split ``all_to_all_single`` moves whole
 slabs, also sync-free.
 """

@@ -32,7 +32,7 @@ def unit_rms(x, eps):
 
 
 def centred_norm(x, w, eps):
-    """RMS norm whose weight is stored around zero."""
+    """RMS norm with a zero-centred weight (applied as 1 + w)."""
     return unit_rms(x, eps) * (1 + w)
 
 
@@ -83,7 +83,7 @@ def rotate_pairs(x, dims: int, base: float):
 
 
 def chunk_sink_attention(h, W, p: str, m: dict):
-    """GQA over the keys of the query's own chunk of positions, softmax with one added to the denominator."""
+    """GQA over the keys of the query's own chunk of positions, softmax whose denominator carries an extra 1."""
     H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     T = h.shape[0]
     proj = {}
