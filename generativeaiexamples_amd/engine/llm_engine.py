@@ -456,7 +456,7 @@ class LLMEngine:
     def _step_done(self) -> None:
         """End of a step on every rank: (followers) wait for the step's GPU work so the staging buffers can
         be reused, then poll the custom all-reduce's error word (RankFailure on a missed peer). Expert-parallel
-        ranks poll their peer-memory all-to-all's error word the same way (ADVICE r4): a peer that died or fell
+        ranks poll their peer-memory all-to-all's error word the same way: a peer that died or fell
         out of lockstep makes the exchange give up after its bounded spin with stale slot data, so the step's
         tokens are invalid; the exchange is retired (later exchanges go to RCCL, its captured graphs are
         dropped) and RankFailure is raised."""
