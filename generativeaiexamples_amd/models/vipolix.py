@@ -153,7 +153,7 @@ class VipolixConfig:
               experts: int = 8, top: int = 2, pattern: Tuple[str, ...] = MIXERS, **kw) -> "VipolixConfig":
         """A regular stack for benchmarks: `pattern` repeated over n_layers; every layer carries `experts` experts of
         ff / top (the active routed feed-forward equals a dense ff) plus a shared expert of ff / 4."""
-        mix = dict(gla=dict(heads=heads, dim=head_dim, vdim=head_dim, tau=16.0),
+        mix = dict(gla=dict(heads=heads, dim=head_dim, vdim=head_dim, tau=8.0),
                    parallel=dict(left=dict(heads=heads, kv_heads=max(1, heads // 4), dim=head_dim, vdim=head_dim, conv=4,
                                            scale=head_dim ** -0.5, mask=dict(size=chunk),
                                            rot=dict(base=10000.0, dims=head_dim // 2)),

@@ -132,7 +132,7 @@ FULL = [O.moe_ff(O.gla()), O.moe_ff(O.par()), O.no_ff(O.par(heads=2, kv_heads=2,
     (O.no_ff(O.gla()), 6), (O.no_ff(O.gla(heads=1, dim=4, vdim=20, tau=1.0)), 0), (O.no_ff(O.gla(heads=5, dim=20, vdim=3, tau=30.0)), 3),
     (O.no_ff(O.par()), 6), (O.no_ff(O.par(heads=3, kv_heads=3, dim=6, vdim=4, conv=1, chunk=1, rot=6, rheads=1, rdim=5)), 0),
     (O.no_ff(O.par(heads=6, kv_heads=1, dim=10, vdim=16, conv=5, chunk=0, rot=0, rheads=3, rdim=12)), 2),
-    (O.no_ff(O.par(heads=2, kv_heads=1, dim=16, vdim=16, conv=0, chunk=64, rot=10, base=250000.0, rheads=2, rdim=16,
+    (O.no_ff(O.par(heads=2, kv_heads=1, dim=16, vdim=16, conv=0, chunk=48, rot=10, base=500000.0, rheads=2, rdim=16,
                    left_scale=1.0, right_scale=1.0)), 6),
     (O.no_ff(O.par(dim=7, vdim=3, rot=2, chunk=16)), 1),
     (O.moe_ff(O.gla()), 6), (O.moe_ff(O.gla(), ff=20, experts=3, top=1, groups=1, keep=1, shared=0), 0),
@@ -140,7 +140,7 @@ FULL = [O.moe_ff(O.gla()), O.moe_ff(O.par()), O.no_ff(O.par(heads=2, kv_heads=2,
     (O.moe_ff(O.par(), ff=24, experts=12, top=3, groups=2, keep=1, scale=2.5), 6),
     (O.moe_ff(O.gla(), ff=16, experts=5, top=5, groups=5, keep=5), 6)],
     ids=["gla", "gla-1head-tau1", "gla-5heads", "parallel", "parallel-mha-chunk1-conv1", "parallel-mqa-causal-norot-conv5",
-         "parallel-noconv-chunk64-part-rotated", "parallel-odd-sizes", "moe", "moe-top1-plain", "moe-8groups-tight-limits",
+         "parallel-noconv-chunk48-part-rotated", "parallel-odd-sizes", "moe", "moe-top1-plain", "moe-8groups-tight-limits",
          "moe-2groups-keep1", "moe-all-experts"])
 def test_single_mechanism(layer, side, device, dtype):
     cfg = config_for(dtype, [layer], width=40, side=side)
@@ -165,7 +165,7 @@ def test_ops_against_oracle_mechanisms(device, dtype):
     z, b = rn(7, 13) * 3, rn(13)
     wide = torch.cat([rn(7, 2), z], 1).to(dev)
     x = z.double() + b.double()
-    for kind, p, want in (("sigmoid", 1.0, torch.sigmoid(x)), ("sigmoid_root", 16.0, torch.sigmoid(x) ** (1 / 16.0)),
+    for kind, p, want in (("sigmoid", 1.0, torch.sigmoid(x)), ("sigmoid_root", 12.0, torch.sigmoid(x) ** (1 / 12.0)),
                           ("sigmoid_root", 0.5, torch.sigmoid(x) ** 2.0), ("exp_sigmoid", O.DECAY_RATE,
                                                                            torch.exp(-O.DECAY_RATE * torch.sigmoid(x)))):
         got = ops.decay_gate(wide[:, 2:], b.to(dev), kind, p).cpu().double()
@@ -344,7 +344,7 @@ def test_far_token_through_state(device, dtype):
     """Slowly forgetting recurrent layers (the attention sees one position): changing four tokens 300 positions back
     changes the last logits (oracle), and the framework follows it, through a prompt cut at odd places and single-token
     steps."""
-    cfg = O.make_config([O.no_ff(O.gla(heads=2, dim=4, vdim=4, tau=16.0)),
+    cfg = O.make_config([O.no_ff(O.gla(heads=2, dim=4, vdim=4, tau=20.0)),
                          O.no_ff(O.par(heads=1, kv_heads=1, dim=4, vdim=4, chunk=1, conv=0, rot=0, rheads=2, rdim=4))],
                         width=32, vocab=64, side=0)
     sd = O.random_checkpoint(cfg, 9, slow_decay=True)
@@ -462,11 +462,11 @@ def test_chunk_edges_bf16_kernels(DK, DV):
 
 @_GPU
 def test_matrix_core_kernels_in_model():
-    """bf16 model with head sizes on the matrix-core grids (attention 64 / 64, expert and projection sizes multiples of
+    """bf16 model with head sizes on the matrix-core grids (attention 64 / 128, expert and projection sizes multiples of
     64): portions of 8+ rows take the matrix-core attention kernel and the MFMA grouped GEMMs, shorter ones and decoded
     tokens the row kernel; both against the oracle, alone and in a mixed batch."""
-    layers = [O.moe_ff(O.par(heads=4, kv_heads=2, dim=64, vdim=64, chunk=48, rot=32, base=10000.0, scale=0.12, rheads=2,
-                             rdim=64), ff=64, experts=4, top=2, groups=2, keep=1, shared=64),
+    layers = [O.moe_ff(O.par(heads=8, kv_heads=2, dim=64, vdim=128, conv=2, chunk=48, rot=16, base=10000.0, scale=0.12,
+                             rheads=2, rdim=64), ff=64, experts=4, top=2, groups=2, keep=1, shared=64),
               O.moe_ff(O.gla(heads=2, dim=64, vdim=64, tau=8.0), ff=128, experts=4, top=2, groups=1, keep=1, shared=0)]
     cfg = config_for(torch.bfloat16, layers, width=128, vocab=128, side=16)
     sd = O.random_checkpoint(cfg, 61)
